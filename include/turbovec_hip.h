@@ -1,0 +1,143 @@
+/*
+ * turbovec_hip.h -- C ABI of the MI355X (gfx950) search path for turbovec.
+ *
+ * The library replaces ONE crate-internal function of the reference,
+ *     search::search(...)                       turbovec/src/search.rs:3206-3221
+ * whose only caller is
+ *     TurboQuantIndex::try_search_with_mask     turbovec/src/lib.rs:1462-1477
+ * plus the small amount of index state that function reads (codes, per-vector
+ * scales, rotation tables, centroids, TQ+ calibration), kept resident in HBM.
+ *
+ * Conventions: every entry point returns a tv_status; nothing throws or aborts
+ * across the boundary; all buffers are caller-owned host memory unless the name
+ * ends in _dev; sizes are element counts.  Functions that mutate an index
+ * (upload / append / swap_remove / set_*) need external exclusion, exactly as
+ * the reference's `&mut self` methods do; tv_search* may be called from many
+ * threads at once (calls on one index are serialised internally).  A process
+ * that has used the library must not fork() and keep using it in the child.
+ */
+#ifndef TURBOVEC_HIP_H
+#define TURBOVEC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tv_index tv_index;
+
+/* Status codes.  1..5 are the reference's SearchError variants
+ * (turbovec/src/error.rs:234-276). */
+typedef enum {
+    TV_OK = 0,
+    TV_ERR_QUERY_BUFFER_NOT_MULTIPLE_OF_DIM = 1, /* lib.rs:1363-1369 */
+    TV_ERR_INVALID_QUERY_VALUE = 2,              /* lib.rs:1374-1380, encode.rs:76-83 */
+    TV_ERR_MASK_LENGTH_MISMATCH = 3,             /* lib.rs:1427-1434 */
+    TV_ERR_ALLOWLIST_EMPTY = 4,                  /* id_map.rs:672 */
+    TV_ERR_UNKNOWN_ID = 5,                       /* id_map.rs:677 */
+    TV_ERR_BAD_ARGUMENT = 6,                     /* ConstructError / FromPartsError class */
+    TV_ERR_HIP = 7,                              /* a HIP runtime call failed */
+    TV_ERR_NO_DEVICE = 8,                        /* no gfx950 device visible */
+    TV_ERR_INDEX_OUT_OF_RANGE = 9
+} tv_status;
+
+/* Which integer score definition the scan uses (the reference picks one at run
+ * time from CPU features, turbovec/src/pack.rs:1189-1219, search.rs:2975-2980). */
+typedef enum {
+    TV_SCORE_AUTO = 0,      /* what an AVX-512 VNNI / dotprod host runs: P at 4-bit, L_U32 at 2/3-bit */
+    TV_SCORE_L_CLASSIC = 2, /* u8 LUT sums, fma flush per 256 byte-groups   search.rs:516-582 */
+    TV_SCORE_L_U32 = 3,     /* u8 LUT sums, (acc*scale+bias)*vec_scale      search.rs:1174-1177 */
+    TV_SCORE_P = 4          /* int8 permute-dot, fma(acc,scale,bias)*vs     search.rs:1519-1524 (4-bit only) */
+} tv_score_mode;
+
+const char *tv_status_string(int status);
+/* Text of the last HIP failure on the calling thread ("" if none). */
+const char *tv_last_error(void);
+
+/* ---- index life cycle -------------------------------------------------- */
+
+/* Replaces the lazily built caches of TurboQuantIndex (lib.rs:1404-1415): the
+ * rotation tables (rotation.rs:141-187) and Lloyd-Max centroids
+ * (codebook.rs:50) are derived inside and uploaded.  dim: positive multiple of
+ * 8, <= 16384; bits in {2,3,4} (lib.rs:629-668).  device: HIP ordinal. */
+int tv_index_create(int dim, int bits, int device, tv_index **out);
+int tv_index_destroy(tv_index *ix);
+
+/* Hand over the caller's own tables instead of the derived ones: signs and
+ * perms are round 0 then round 1 (2*dim each, rotation.rs:110-115), centroids
+ * 2^bits values.  Any pointer may be NULL to keep the current table. */
+int tv_index_set_tables(tv_index *ix, const float *signs, const uint32_t *perms, const float *centroids);
+/* TQ+ pair (lib.rs:329-330), dim values each; both NULL = uncalibrated. */
+int tv_index_set_calibration(tv_index *ix, const float *shift, const float *scale);
+int tv_index_set_score_mode(tv_index *ix, int mode);
+
+/* Read back the tables in use (for cross-checking against the caller's). */
+int tv_index_get_tables(const tv_index *ix, float *signs, uint32_t *perms, float *centroids, float *boundaries);
+
+/* Replace the contents with n_vectors rows given in the sequential-blocked
+ * layout the reference persists (pack.rs:336-361: byte of (block b, group g,
+ * lane l) at (b*G+g)*32+l, ceil(n/32)*G*32 bytes) and their per-vector scales
+ * (lib.rs:312).  Replaces BlockedCache (lib.rs:253-256). */
+int tv_index_upload_seq(tv_index *ix, const uint8_t *seq_codes, size_t n_vectors, const float *scales);
+/* Append n_new rows; rows[i*G + g] is row i's code byte of group g (the
+ * per-vector form extract_codes_flat yields, pack.rs:306).  Replaces
+ * append_lanes (pack.rs:211-233). */
+int tv_index_append_rows(tv_index *ix, const uint8_t *rows, const float *scales, size_t n_new);
+/* lib.rs:2864-3028: move the last vector into slot idx, zero the vacated lane. */
+int tv_index_swap_remove(tv_index *ix, size_t idx);
+/* Copy the index back in the sequential-blocked layout (codes_blocked_seq,
+ * lib.rs:2088); seq_out holds ceil(n/32)*G*32 bytes, scales_out n floats. */
+int tv_index_download_seq(const tv_index *ix, uint8_t *seq_out, float *scales_out);
+size_t tv_index_len(const tv_index *ix);
+int tv_index_dim(const tv_index *ix);
+int tv_index_bits(const tv_index *ix);
+
+/* ---- search ------------------------------------------------------------- */
+
+/* Caller-side validation the reference performs before the seam
+ * (lib.rs:1363-1380): len must be a multiple of dim, every value must satisfy
+ * |x| < 1e16.  On TV_ERR_INVALID_QUERY_VALUE *bad_index is the flat offset. */
+int tv_validate_queries(const float *queries, size_t len, int dim, size_t *bad_index);
+/* lib.rs:1435-1456: one byte per slot (non-zero = allowed) to u64 words, LSB =
+ * lowest slot; returns the number of allowed slots in *n_allowed. */
+int tv_pack_mask(const uint8_t *mask_bytes, size_t n, uint64_t *words_out, size_t *n_allowed);
+
+/* search::search (search.rs:3206).  queries: nq*dim floats.  mask_words: NULL
+ * or ceil(n/64) words.  Writes nq*k_eff scores and slot indices, rows sorted
+ * (score desc, slot asc), k_eff = min(k, n, popcount(mask)) returned in
+ * *out_k_eff; out buffers must hold nq*min(k,n) entries.  k_eff == 0 or
+ * nq == 0 writes nothing. */
+int tv_search(tv_index *ix, const float *queries, size_t nq, size_t k,
+              const uint64_t *mask_words, size_t n_mask_words,
+              float *out_scores, int64_t *out_indices, size_t *out_k_eff);
+
+/* Same, with queries, mask words and outputs already in device memory and the
+ * mask's popcount supplied by the caller (the reference's caller counts it
+ * while packing, lib.rs:1446).  Returns after the work is enqueued and
+ * completed on the index's stream. */
+int tv_search_dev(tv_index *ix, const float *d_queries, size_t nq, size_t k,
+                  const uint64_t *d_mask_words, size_t n_allowed,
+                  float *d_out_scores, int64_t *d_out_indices, size_t *out_k_eff);
+
+/* ---- test / measurement hooks -------------------------------------------- */
+
+/* Integer accumulators and final float scores of every (query, slot) pair,
+ * nq*n each (either may be NULL): what the parity tests compare bit-for-bit. */
+int tv_debug_scan(tv_index *ix, const float *queries, size_t nq, int32_t *acc_out, float *scores_out);
+/* Query preparation only: rotated (and TQ+-calibrated) rows nq*dim, and per
+ * query scale and bias of the active score mode (any may be NULL). */
+int tv_debug_prepare(tv_index *ix, const float *queries, size_t nq,
+                     float *q_rot_out, float *scale_out, float *bias_out);
+/* Duration in milliseconds of the scan kernel launches of the most recent
+ * tv_search* call on this index, measured with HIP events on its stream, and
+ * how many launches that was. */
+int tv_last_scan_ms(const tv_index *ix, float *ms, int *launches);
+/* Device pointers of the resident index (native layout) for tools. */
+int tv_index_device_ptrs(const tv_index *ix, void **d_codes, void **d_scales, size_t *code_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

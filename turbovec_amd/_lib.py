@@ -1,0 +1,228 @@
+"""ctypes binding of libturbovec_hip.so (the C ABI declared in include/turbovec_hip.h).
+
+There is no CPU fallback: if the library is missing or a call fails, this raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libturbovec_hip.so")
+
+OK = 0
+ERR_QUERY_BUFFER_NOT_MULTIPLE_OF_DIM = 1
+ERR_INVALID_QUERY_VALUE = 2
+ERR_MASK_LENGTH_MISMATCH = 3
+ERR_ALLOWLIST_EMPTY = 4
+ERR_UNKNOWN_ID = 5
+ERR_BAD_ARGUMENT = 6
+ERR_HIP = 7
+ERR_NO_DEVICE = 8
+ERR_INDEX_OUT_OF_RANGE = 9
+
+SCORE_AUTO, SCORE_L_CLASSIC, SCORE_L_U32, SCORE_P = 0, 2, 3, 4
+
+# every symbol include/turbovec_hip.h declares
+EXPORTS = [
+    "tv_status_string", "tv_last_error", "tv_index_create", "tv_index_destroy", "tv_index_set_tables",
+    "tv_index_set_calibration", "tv_index_set_score_mode", "tv_index_get_tables", "tv_index_upload_seq",
+    "tv_index_append_rows", "tv_index_swap_remove", "tv_index_download_seq", "tv_index_len", "tv_index_dim",
+    "tv_index_bits", "tv_validate_queries", "tv_pack_mask", "tv_search", "tv_search_dev", "tv_debug_scan",
+    "tv_debug_prepare", "tv_last_scan_ms", "tv_index_device_ptrs",
+]
+
+_lib = None
+
+
+class TurbovecHipError(RuntimeError):
+    def __init__(self, status, detail=""):
+        self.status = status
+        super().__init__(f"turbovec_hip status {status}: {detail}")
+
+
+def lib():
+    """Load the built library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m turbovec_amd.build` (hipcc, gfx950). "
+            "The search path has no CPU fallback.")
+    L = C.CDLL(LIB_PATH)
+    vp, sz, i32 = C.c_void_p, C.c_size_t, C.c_int
+    L.tv_status_string.restype = C.c_char_p
+    L.tv_status_string.argtypes = [i32]
+    L.tv_last_error.restype = C.c_char_p
+    L.tv_index_create.argtypes = [i32, i32, i32, C.POINTER(vp)]
+    L.tv_index_destroy.argtypes = [vp]
+    L.tv_index_set_tables.argtypes = [vp, vp, vp, vp]
+    L.tv_index_set_calibration.argtypes = [vp, vp, vp]
+    L.tv_index_set_score_mode.argtypes = [vp, i32]
+    L.tv_index_get_tables.argtypes = [vp, vp, vp, vp, vp]
+    L.tv_index_upload_seq.argtypes = [vp, vp, sz, vp]
+    L.tv_index_append_rows.argtypes = [vp, vp, vp, sz]
+    L.tv_index_swap_remove.argtypes = [vp, sz]
+    L.tv_index_download_seq.argtypes = [vp, vp, vp]
+    L.tv_index_len.restype = sz
+    L.tv_index_len.argtypes = [vp]
+    L.tv_index_dim.argtypes = [vp]
+    L.tv_index_bits.argtypes = [vp]
+    L.tv_validate_queries.argtypes = [vp, sz, i32, C.POINTER(sz)]
+    L.tv_pack_mask.argtypes = [vp, sz, vp, C.POINTER(sz)]
+    L.tv_search.argtypes = [vp, vp, sz, sz, vp, sz, vp, vp, C.POINTER(sz)]
+    L.tv_search_dev.argtypes = [vp, vp, sz, sz, vp, sz, vp, vp, C.POINTER(sz)]
+    L.tv_debug_scan.argtypes = [vp, vp, sz, vp, vp]
+    L.tv_debug_prepare.argtypes = [vp, vp, sz, vp, vp, vp]
+    L.tv_last_scan_ms.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(i32)]
+    L.tv_index_device_ptrs.argtypes = [vp, C.POINTER(vp), C.POINTER(vp), C.POINTER(sz)]
+    _lib = L
+    return L
+
+
+def check(status):
+    if status != OK:
+        L = lib()
+        detail = L.tv_status_string(status).decode()
+        extra = L.tv_last_error().decode()
+        raise TurbovecHipError(status, detail + (": " + extra if extra else ""))
+
+
+def ptr(a):
+    return None if a is None else a.ctypes.data
+
+
+class NativeIndex:
+    """Thin owner of a tv_index handle (device-resident codes, scales and tables)."""
+
+    def __init__(self, dim, bits, device=0):
+        h = C.c_void_p()
+        check(lib().tv_index_create(dim, bits, device, C.byref(h)))
+        self.h = h
+        self.dim, self.bits = dim, bits
+        self.n_byte_groups = dim // (8 // bits)
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().tv_index_destroy(self.h)
+            self.h = None
+
+    __del__ = close
+
+    def __len__(self):
+        return lib().tv_index_len(self.h)
+
+    def set_score_mode(self, mode):
+        check(lib().tv_index_set_score_mode(self.h, mode))
+
+    def set_calibration(self, shift, scale):
+        if shift is None:
+            check(lib().tv_index_set_calibration(self.h, None, None))
+            return
+        sh = np.ascontiguousarray(shift, np.float32)
+        sc = np.ascontiguousarray(scale, np.float32)
+        assert sh.shape == (self.dim,) and sc.shape == (self.dim,)
+        check(lib().tv_index_set_calibration(self.h, ptr(sh), ptr(sc)))
+
+    def set_tables(self, signs=None, perms=None, centroids=None):
+        s = None if signs is None else np.ascontiguousarray(signs, np.float32)
+        p = None if perms is None else np.ascontiguousarray(perms, np.uint32)
+        c = None if centroids is None else np.ascontiguousarray(centroids, np.float32)
+        check(lib().tv_index_set_tables(self.h, ptr(s), ptr(p), ptr(c)))
+
+    def tables(self):
+        signs = np.zeros((2, self.dim), np.float32)
+        perms = np.zeros((2, self.dim), np.uint32)
+        cen = np.zeros(1 << self.bits, np.float32)
+        bnd = np.zeros((1 << self.bits) - 1, np.float32)
+        check(lib().tv_index_get_tables(self.h, ptr(signs), ptr(perms), ptr(cen), ptr(bnd)))
+        return signs, perms, cen, bnd
+
+    def upload_seq(self, seq_codes, n, scales):
+        seq = np.ascontiguousarray(seq_codes, np.uint8)
+        sc = np.ascontiguousarray(scales, np.float32)
+        assert seq.size == ((n + 31) // 32) * self.n_byte_groups * 32, "sequential-blocked size mismatch"
+        assert sc.size == n
+        check(lib().tv_index_upload_seq(self.h, ptr(seq), n, ptr(sc)))
+
+    def append_rows(self, rows, scales):
+        r = np.ascontiguousarray(rows, np.uint8).reshape(-1, self.n_byte_groups)
+        sc = np.ascontiguousarray(scales, np.float32)
+        assert len(sc) == len(r)
+        check(lib().tv_index_append_rows(self.h, ptr(r), ptr(sc), len(r)))
+
+    def swap_remove(self, idx):
+        check(lib().tv_index_swap_remove(self.h, idx))
+
+    def download_seq(self):
+        n = len(self)
+        seq = np.zeros(((n + 31) // 32) * self.n_byte_groups * 32, np.uint8)
+        sc = np.zeros(n, np.float32)
+        check(lib().tv_index_download_seq(self.h, ptr(seq), ptr(sc)))
+        return seq, sc
+
+    def search(self, queries, k, mask_words=None):
+        q = np.ascontiguousarray(queries, np.float32).reshape(-1, self.dim)
+        nq = q.shape[0]
+        n = len(self)
+        cap = min(k, n)
+        out_s = np.zeros((nq, cap), np.float32)
+        out_i = np.zeros((nq, cap), np.int64)
+        k_eff = C.c_size_t(0)
+        mw = None if mask_words is None else np.ascontiguousarray(mask_words, np.uint64)
+        check(lib().tv_search(self.h, ptr(q), nq, k, ptr(mw), 0 if mw is None else mw.size, ptr(out_s), ptr(out_i),
+                              C.byref(k_eff)))
+        ke = k_eff.value
+        if ke == cap:
+            return out_s, out_i
+        return (np.ascontiguousarray(out_s.ravel()[: nq * ke].reshape(nq, ke)),
+                np.ascontiguousarray(out_i.ravel()[: nq * ke].reshape(nq, ke)))
+
+    def search_dev(self, d_queries_ptr, nq, k, d_out_scores_ptr, d_out_idx_ptr, d_mask_ptr=None, n_allowed=0):
+        k_eff = C.c_size_t(0)
+        check(lib().tv_search_dev(self.h, d_queries_ptr, nq, k, d_mask_ptr, n_allowed, d_out_scores_ptr,
+                                  d_out_idx_ptr, C.byref(k_eff)))
+        return k_eff.value
+
+    def debug_scan(self, queries):
+        q = np.ascontiguousarray(queries, np.float32).reshape(-1, self.dim)
+        n = len(self)
+        acc = np.zeros((q.shape[0], n), np.int32)
+        sc = np.zeros((q.shape[0], n), np.float32)
+        check(lib().tv_debug_scan(self.h, ptr(q), q.shape[0], ptr(acc), ptr(sc)))
+        return acc, sc
+
+    def debug_prepare(self, queries):
+        q = np.ascontiguousarray(queries, np.float32).reshape(-1, self.dim)
+        rot = np.zeros_like(q)
+        scale = np.zeros(q.shape[0], np.float32)
+        bias = np.zeros(q.shape[0], np.float32)
+        check(lib().tv_debug_prepare(self.h, ptr(q), q.shape[0], ptr(rot), ptr(scale), ptr(bias)))
+        return rot, scale, bias
+
+    def last_scan_ms(self):
+        ms = C.c_float(0)
+        n = C.c_int(0)
+        check(lib().tv_last_scan_ms(self.h, C.byref(ms), C.byref(n)))
+        return ms.value, n.value
+
+    def device_ptrs(self):
+        a, b, s = C.c_void_p(), C.c_void_p(), C.c_size_t()
+        check(lib().tv_index_device_ptrs(self.h, C.byref(a), C.byref(b), C.byref(s)))
+        return a.value, b.value, s.value
+
+
+def validate_queries(queries_flat, dim):
+    q = np.ascontiguousarray(queries_flat, np.float32).ravel()
+    bad = C.c_size_t(0)
+    rc = lib().tv_validate_queries(ptr(q), q.size, dim, C.byref(bad))
+    return rc, bad.value
+
+
+def pack_mask(mask_bytes):
+    m = np.ascontiguousarray(mask_bytes).view(np.uint8).ravel()
+    words = np.zeros((m.size + 63) // 64, np.uint64)
+    allowed = C.c_size_t(0)
+    check(lib().tv_pack_mask(ptr(m), m.size, ptr(words), C.byref(allowed)))
+    return words, allowed.value

@@ -1,0 +1,681 @@
+// C ABI of the search path (see include/turbovec_hip.h).
+#include "../../include/turbovec_hip.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+
+#include "tv_internal.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail_hip(hipError_t e, const char *what) {
+    char buf[256];
+    snprintf(buf, sizeof buf, "%s: %s", what, hipGetErrorString(e));
+    g_last_error = buf;
+    return TV_ERR_HIP;
+}
+
+#define TV_HIP(call)                                        \
+    do {                                                    \
+        hipError_t e__ = (call);                            \
+        if (e__ != hipSuccess) return fail_hip(e__, #call); \
+    } while (0)
+
+size_t round_up(size_t v, size_t m) { return (v + m - 1) / m * m; }
+
+// Bump allocator over the index's cached workspace.
+struct Arena {
+    uint8_t *base = nullptr;
+    size_t used = 0;
+    template <typename T>
+    T *take(size_t count) {
+        T *p = reinterpret_cast<T *>(base + used);
+        used += round_up(count * sizeof(T), 256);
+        return p;
+    }
+};
+
+int ensure_workspace(tv_index *ix, size_t bytes) {
+    if (bytes <= ix->ws_bytes) return TV_OK;
+    if (ix->ws) { TV_HIP(hipFree(ix->ws)); ix->ws = nullptr; ix->ws_bytes = 0; }
+    bytes = round_up(bytes + bytes / 4, size_t(1) << 20);
+    TV_HIP(hipMalloc(&ix->ws, bytes));
+    ix->ws_bytes = bytes;
+    return TV_OK;
+}
+
+int ensure_capacity(tv_index *ix, size_t n_vectors) {
+    const size_t blocks = (n_vectors + tv::kVecBlock - 1) / tv::kVecBlock;
+    if (blocks <= ix->cap_blocks) return TV_OK;
+    size_t cap = std::max(blocks, ix->cap_blocks + ix->cap_blocks / 2);
+    cap = std::max<size_t>(cap, 64);
+    uint8_t *codes = nullptr;
+    float *scales = nullptr;
+    const size_t bb = ix->geo.block_bytes();
+    TV_HIP(hipMalloc(reinterpret_cast<void **>(&codes), cap * bb));
+    TV_HIP(hipMalloc(reinterpret_cast<void **>(&scales), cap * tv::kVecBlock * sizeof(float)));
+    const size_t old_blocks = (ix->n + tv::kVecBlock - 1) / tv::kVecBlock;
+    // fresh bytes are zero so padding lanes match a from-scratch upload
+    TV_HIP(hipMemsetAsync(codes + old_blocks * bb, 0, (cap - old_blocks) * bb, ix->stream));
+    TV_HIP(hipMemsetAsync(scales + old_blocks * tv::kVecBlock, 0,
+                          (cap - old_blocks) * tv::kVecBlock * sizeof(float), ix->stream));
+    if (old_blocks) {
+        TV_HIP(hipMemcpyAsync(codes, ix->d_codes, old_blocks * bb, hipMemcpyDeviceToDevice, ix->stream));
+        TV_HIP(hipMemcpyAsync(scales, ix->d_scales, old_blocks * tv::kVecBlock * sizeof(float),
+                              hipMemcpyDeviceToDevice, ix->stream));
+    }
+    TV_HIP(hipStreamSynchronize(ix->stream));
+    if (ix->d_codes) TV_HIP(hipFree(ix->d_codes));
+    if (ix->d_scales) TV_HIP(hipFree(ix->d_scales));
+    ix->d_codes = codes;
+    ix->d_scales = scales;
+    ix->cap_blocks = cap;
+    return TV_OK;
+}
+
+// turbovec/src/search.rs:2812-2820: the codebook as int8 levels, one scale.
+void derive_levels(tv_index *ix) {
+    float cmax = 0.0f;
+    for (float c : ix->cb.centroids) cmax = std::fmax(cmax, std::fabs(c));
+    ix->cs = cmax > 0.0f ? cmax / 127.0f : 1.0f;
+    std::memset(ix->levels, 0, sizeof ix->levels);
+    for (size_t i = 0; i < ix->cb.centroids.size() && i < 16; ++i) {
+        float v = std::round(ix->cb.centroids[i] / ix->cs);
+        v = v < -127.0f ? -127.0f : (v > 127.0f ? 127.0f : v);
+        ix->levels[i] = int8_t(v);
+    }
+}
+
+int upload_tables(tv_index *ix) {
+    const size_t dim = size_t(ix->geo.dim);
+    TV_HIP(hipMemcpyAsync(ix->d_signs, ix->rot.signs.data(), 2 * dim * sizeof(float), hipMemcpyHostToDevice,
+                          ix->stream));
+    TV_HIP(hipMemcpyAsync(ix->d_perms, ix->rot.perms.data(), 2 * dim * sizeof(uint32_t), hipMemcpyHostToDevice,
+                          ix->stream));
+    float cen[16] = {0};
+    for (size_t i = 0; i < ix->cb.centroids.size(); ++i) cen[i] = ix->cb.centroids[i];
+    TV_HIP(hipMemcpyAsync(ix->d_centroids, cen, sizeof cen, hipMemcpyHostToDevice, ix->stream));
+    TV_HIP(hipStreamSynchronize(ix->stream));
+    return TV_OK;
+}
+
+int effective_mode(const tv_index *ix) {
+    int m = ix->score_mode;
+    if (m == TV_SCORE_AUTO) m = ix->geo.bits == 4 ? TV_SCORE_P : TV_SCORE_L_U32;
+    return m;
+}
+
+struct Prepared {
+    float *d_qrot = nullptr;   // rotated (and calibrated) rows
+    uint8_t *d_tables = nullptr;
+    float *d_qscale = nullptr, *d_qbias = nullptr;
+    size_t table_bytes_per_tile = 0;
+};
+
+// Query preparation for one chunk: rotation, TQ+ inverse, table build
+// (turbovec/src/search.rs:3237-3269).  d_q holds nq*dim floats on the device.
+int prepare_queries(tv_index *ix, Arena &ar, const float *d_q, size_t nq, Prepared &out) {
+    const tv::Geometry &g = ix->geo;
+    const size_t nq_pad = round_up(nq, tv::kQTile);
+    const int mode = effective_mode(ix);
+    float *d_rot = ar.take<float>(nq * g.dim);
+    float *d_bias_corr = ar.take<float>(nq_pad);
+    TV_HIP(tv::launch_rotate(d_q, d_rot, ix->d_signs, ix->d_perms, g.dim, ix->rot.block, ix->rot.inv_sqrt_block, nq,
+                             ix->stream));
+    float *d_cal = d_rot;
+    if (!ix->tq_shift.empty()) {
+        d_cal = ar.take<float>(nq * g.dim);
+        TV_HIP(tv::launch_calibrate(d_rot, d_cal, d_bias_corr, ix->d_tq_shift, ix->d_tq_scale, g.dim, nq,
+                                    ix->stream));
+    } else {
+        TV_HIP(tv::launch_fill_i32(reinterpret_cast<int *>(d_bias_corr), 0, nq_pad, ix->stream));
+    }
+    out.d_qrot = d_cal;
+    out.d_qscale = ar.take<float>(nq_pad);
+    out.d_qbias = ar.take<float>(nq_pad);
+    if (mode == TV_SCORE_P) {
+        out.table_bytes_per_tile = size_t(g.nch) * 2048;
+        out.d_tables = ar.take<uint8_t>(nq_pad / tv::kQTile * out.table_bytes_per_tile);
+        TV_HIP(tv::launch_build_p(d_cal, d_bias_corr, out.d_tables, out.d_qscale, out.d_qbias, g.dim, g.G, g.nch,
+                                  ix->cs, nq, nq_pad, ix->stream));
+    } else {
+        out.table_bytes_per_tile = size_t(g.nch) * 1024 * tv::kQTile;
+        out.d_tables = ar.take<uint8_t>(nq_pad * size_t(g.nch) * 1024);
+        TV_HIP(tv::launch_build_lut(d_cal, d_bias_corr, ix->d_centroids, out.d_tables, out.d_qscale, out.d_qbias,
+                                    g.dim, g.bits, g.G, g.nch, nq, nq_pad, ix->stream));
+    }
+    return TV_OK;
+}
+
+size_t prepare_bytes(const tv_index *ix, size_t nq) {
+    const tv::Geometry &g = ix->geo;
+    const size_t nq_pad = round_up(nq, tv::kQTile);
+    size_t b = 2 * round_up(nq * g.dim * 4, 256) + 3 * round_up(nq_pad * 4, 256);
+    b += round_up(nq_pad * size_t(g.nch) * 1024, 256) + 4096;
+    return b;
+}
+
+void fill_scan_args(const tv_index *ix, tv::ScanArgs &a) {
+    std::memset(&a, 0, sizeof a);
+    a.codes = ix->d_codes;
+    a.scales = ix->d_scales;
+    a.n = uint32_t(ix->n);
+    a.n_blocks = uint32_t((ix->n + tv::kVecBlock - 1) / tv::kVecBlock);
+    a.nch = ix->geo.nch;
+    std::memcpy(a.lv, ix->levels, 16);
+    a.classic = effective_mode(ix) == TV_SCORE_L_CLASSIC;
+}
+
+constexpr size_t kChunkQueries = 4096;
+constexpr int kMaxTimedTiles = int(kChunkQueries / tv::kQTile);
+
+struct EventPool {
+    hipEvent_t start[kMaxTimedTiles];
+    hipEvent_t stop[kMaxTimedTiles];
+    bool ready = false;
+};
+thread_local EventPool g_events;
+
+int ensure_events() {
+    if (g_events.ready) return TV_OK;
+    for (int i = 0; i < kMaxTimedTiles; ++i) {
+        TV_HIP(hipEventCreate(&g_events.start[i]));
+        TV_HIP(hipEventCreate(&g_events.stop[i]));
+    }
+    g_events.ready = true;
+    return TV_OK;
+}
+
+// The seam: search::search over device-resident inputs and outputs.
+int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, const uint64_t *d_mask,
+                  size_t n_allowed, float *d_out_scores, int64_t *d_out_idx, size_t *out_k_eff) {
+    const size_t n = ix->n;
+    size_t k_eff = std::min(std::min(k, n), n_allowed);  // lib.rs:1460, search.rs:3222-3225
+    if (out_k_eff) *out_k_eff = k_eff;
+    ix->last_scan_ms = 0.0f;
+    ix->last_scan_launches = 0;
+    if (k_eff == 0 || nq == 0) return TV_OK;                // search.rs:3226-3229
+    if (n >= (size_t(1) << 31)) { g_last_error = "index too large for 31-bit slots"; return TV_ERR_BAD_ARGUMENT; }
+    const tv::Geometry &g = ix->geo;
+    const int mode = effective_mode(ix);
+    if (mode == TV_SCORE_P && g.bits != 4) { g_last_error = "score mode P needs 4-bit codes"; return TV_ERR_BAD_ARGUMENT; }
+    const bool mode_p = mode == TV_SCORE_P;
+    const bool lists = k_eff <= size_t(tv::kMaxListK);
+    int rc = ensure_events();
+    if (rc != TV_OK) return rc;
+
+    for (size_t q0 = 0; q0 < nq; q0 += kChunkQueries) {
+        const size_t cq = std::min(kChunkQueries, nq - q0);
+        const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_tile_queries(g.nch, lists ? int(k_eff) : 1));
+        const size_t n_tiles = (cq + tile_q - 1) / tile_q;
+        const int grid = tv::scan_grid_blocks(ix->device, mode_p, g.nch, lists ? int(k_eff) : 1, int(tile_q));
+        const size_t total_threads = size_t(grid) * tv::kScanThreads;
+        size_t need = prepare_bytes(ix, cq) + round_up(n_tiles * tv::kQTile * 4, 256);
+        if (lists) need += 2 * round_up(k_eff * total_threads * 4, 256) + round_up(total_threads * 4, 256);
+        else need += round_up(size_t(tv::kQTile) * n * 4, 256) + round_up(tv::select_tmp_keys(k_eff) * 8 * tv::kQTile, 256) +
+                     round_up(size_t(tv::kQTile) * 4096 * 4, 256);
+        rc = ensure_workspace(ix, need + 65536);
+        if (rc != TV_OK) return rc;
+        Arena ar;
+        ar.base = static_cast<uint8_t *>(ix->ws);
+        Prepared pq;
+        rc = prepare_queries(ix, ar, d_queries + q0 * g.dim, cq, pq);
+        if (rc != TV_OK) return rc;
+        int *d_tau = ar.take<int>(n_tiles * tv::kQTile);
+        TV_HIP(tv::launch_fill_i32(d_tau, int(0x807fffffu) /* order key of -inf */, n_tiles * tv::kQTile, ix->stream));
+        float *d_part_s = nullptr, *d_dense = nullptr;
+        uint32_t *d_part_i = nullptr, *d_hist = nullptr;
+        int *d_part_c = nullptr;
+        uint64_t *d_keys = nullptr;
+        if (lists) {
+            d_part_s = ar.take<float>(k_eff * total_threads);
+            d_part_i = ar.take<uint32_t>(k_eff * total_threads);
+            d_part_c = ar.take<int>(total_threads);
+        } else {
+            d_dense = ar.take<float>(size_t(tv::kQTile) * n);
+            d_keys = ar.take<uint64_t>(tv::select_tmp_keys(k_eff) * tv::kQTile);
+            d_hist = ar.take<uint32_t>(size_t(tv::kQTile) * 4096);
+        }
+        for (size_t t = 0; t < n_tiles; ++t) {
+            tv::ScanArgs a;
+            fill_scan_args(ix, a);
+            a.mask = d_mask;
+            a.tables = pq.d_tables + t * (mode_p ? pq.table_bytes_per_tile : tile_q * size_t(g.nch) * 1024);
+            a.qscale = pq.d_qscale + t * tile_q;
+            a.qbias = pq.d_qbias + t * tile_q;
+            a.nq_tile = int(std::min<size_t>(tile_q, cq - t * tile_q));
+            a.k = int(lists ? k_eff : 1);
+            a.gtau = d_tau + t * tv::kQTile;
+            a.part_scores = d_part_s; a.part_idx = d_part_i; a.part_cnt = d_part_c;
+            a.score_out = d_dense;
+            if (!lists && d_mask) // blocks without an allowed slot are skipped by the scan: mark them excluded
+                TV_HIP(tv::launch_fill_i32(reinterpret_cast<int *>(d_dense), 0x7fc00000, size_t(a.nq_tile) * n, ix->stream));
+            const bool timed = int(t) < kMaxTimedTiles;
+            if (timed) TV_HIP(hipEventRecord(g_events.start[t], ix->stream));
+            if (mode_p) TV_HIP(tv::launch_scan_p4(a, grid, !lists, ix->stream));
+            else TV_HIP(tv::launch_scan_lut(a, grid, !lists, ix->stream));
+            if (timed) TV_HIP(hipEventRecord(g_events.stop[t], ix->stream));
+            float *os = d_out_scores + (q0 + t * tile_q) * k_eff;
+            int64_t *oi = d_out_idx + (q0 + t * tile_q) * k_eff;
+            if (lists) {
+                const int qmod = mode_p ? tv::kQTile : tv::lut_launch_ql(g.nch, int(k_eff), a.nq_tile);
+                TV_HIP(tv::launch_merge(d_part_s, d_part_i, d_part_c, int(total_threads), qmod, int(k_eff), int(k_eff),
+                                        a.nq_tile, os, oi, ix->stream));
+            } else {
+                TV_HIP(tv::launch_select_topk(d_dense, n, a.nq_tile, k_eff, d_keys, d_hist, os, oi, ix->stream));
+            }
+        }
+        TV_HIP(hipStreamSynchronize(ix->stream));
+        for (size_t t = 0; t < n_tiles && int(t) < kMaxTimedTiles; ++t) {
+            float ms = 0.0f;
+            TV_HIP(hipEventElapsedTime(&ms, g_events.start[t], g_events.stop[t]));
+            ix->last_scan_ms += ms;
+            ix->last_scan_launches += 1;
+        }
+    }
+    return TV_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *tv_status_string(int status) {
+    switch (status) {
+        case TV_OK: return "ok";
+        case TV_ERR_QUERY_BUFFER_NOT_MULTIPLE_OF_DIM: return "query buffer length not a multiple of dim";
+        case TV_ERR_INVALID_QUERY_VALUE: return "invalid query value (must be finite and |value| < 1e16)";
+        case TV_ERR_MASK_LENGTH_MISMATCH: return "mask length does not match index size";
+        case TV_ERR_ALLOWLIST_EMPTY: return "allowlist is empty";
+        case TV_ERR_UNKNOWN_ID: return "id in allowlist is not present in index";
+        case TV_ERR_BAD_ARGUMENT: return "bad argument";
+        case TV_ERR_HIP: return "HIP runtime error";
+        case TV_ERR_NO_DEVICE: return "no usable GPU";
+        case TV_ERR_INDEX_OUT_OF_RANGE: return "index out of range";
+        default: return "unknown status";
+    }
+}
+
+const char *tv_last_error(void) { return g_last_error.c_str(); }
+
+int tv_index_create(int dim, int bits, int device, tv_index **out) {
+    if (!out) return TV_ERR_BAD_ARGUMENT;
+    *out = nullptr;
+    if (bits < 2 || bits > 4) { g_last_error = "bit_width must be 2, 3, or 4"; return TV_ERR_BAD_ARGUMENT; }
+    if (dim <= 0 || dim % 8 != 0) { g_last_error = "dim must be a positive multiple of 8"; return TV_ERR_BAD_ARGUMENT; }
+    if (dim > 16384) { g_last_error = "dim exceeds maximum 16384"; return TV_ERR_BAD_ARGUMENT; }
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= device || device < 0) {
+        g_last_error = "no HIP device with that ordinal";
+        return TV_ERR_NO_DEVICE;
+    }
+    TV_HIP(hipSetDevice(device));
+    tv_index *ix = new (std::nothrow) tv_index();
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    ix->device = device;
+    ix->geo.dim = dim;
+    ix->geo.bits = bits;
+    ix->geo.G = dim / (8 / bits);
+    ix->geo.nch = (ix->geo.G + tv::kChunkGroups - 1) / tv::kChunkGroups;
+    ix->rot = tv::make_rotation_tables(dim);
+    ix->cb = tv::make_codebook(bits, dim);
+    derive_levels(ix);
+    int rc = TV_OK;
+    do {
+        if (hipStreamCreateWithFlags(&ix->stream, hipStreamNonBlocking) != hipSuccess) { rc = TV_ERR_HIP; break; }
+        if (hipMalloc(reinterpret_cast<void **>(&ix->d_signs), 2 * size_t(dim) * sizeof(float)) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void **>(&ix->d_perms), 2 * size_t(dim) * sizeof(uint32_t)) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void **>(&ix->d_centroids), 16 * sizeof(float)) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void **>(&ix->d_tq_shift), size_t(dim) * sizeof(float)) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void **>(&ix->d_tq_scale), size_t(dim) * sizeof(float)) != hipSuccess) {
+            rc = TV_ERR_HIP;
+            break;
+        }
+        rc = upload_tables(ix);
+    } while (0);
+    if (rc != TV_OK) {
+        if (g_last_error.empty()) g_last_error = "device allocation failed";
+        tv_index_destroy(ix);
+        return rc;
+    }
+    *out = ix;
+    return TV_OK;
+}
+
+int tv_index_destroy(tv_index *ix) {
+    if (!ix) return TV_OK;
+    (void)hipSetDevice(ix->device);
+    if (ix->stream) (void)hipStreamSynchronize(ix->stream);
+    void *ptrs[] = {ix->d_signs, ix->d_perms, ix->d_centroids, ix->d_tq_shift, ix->d_tq_scale,
+                    ix->d_codes, ix->d_scales, ix->ws};
+    for (void *p : ptrs) if (p) (void)hipFree(p);
+    if (ix->stream) (void)hipStreamDestroy(ix->stream);
+    delete ix;
+    return TV_OK;
+}
+
+int tv_index_set_tables(tv_index *ix, const float *signs, const uint32_t *perms, const float *centroids) {
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    TV_HIP(hipSetDevice(ix->device));
+    const size_t dim = size_t(ix->geo.dim);
+    if (signs) ix->rot.signs.assign(signs, signs + 2 * dim);
+    if (perms) {
+        for (size_t i = 0; i < 2 * dim; ++i) if (perms[i] >= dim) return TV_ERR_BAD_ARGUMENT;
+        ix->rot.perms.assign(perms, perms + 2 * dim);
+    }
+    if (centroids) {
+        ix->cb.centroids.assign(centroids, centroids + (size_t(1) << ix->geo.bits));
+        for (size_t i = 0; i + 1 < ix->cb.centroids.size(); ++i)
+            ix->cb.boundaries[i] = (ix->cb.centroids[i] + ix->cb.centroids[i + 1]) * 0.5f;
+        derive_levels(ix);
+    }
+    return upload_tables(ix);
+}
+
+int tv_index_set_calibration(tv_index *ix, const float *shift, const float *scale) {
+    if (!ix || (shift == nullptr) != (scale == nullptr)) return TV_ERR_BAD_ARGUMENT;
+    TV_HIP(hipSetDevice(ix->device));
+    const size_t dim = size_t(ix->geo.dim);
+    if (!shift) { ix->tq_shift.clear(); ix->tq_scale.clear(); return TV_OK; }
+    ix->tq_shift.assign(shift, shift + dim);
+    ix->tq_scale.assign(scale, scale + dim);
+    TV_HIP(hipMemcpyAsync(ix->d_tq_shift, shift, dim * sizeof(float), hipMemcpyHostToDevice, ix->stream));
+    TV_HIP(hipMemcpyAsync(ix->d_tq_scale, scale, dim * sizeof(float), hipMemcpyHostToDevice, ix->stream));
+    TV_HIP(hipStreamSynchronize(ix->stream));
+    return TV_OK;
+}
+
+int tv_index_set_score_mode(tv_index *ix, int mode) {
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    if (mode != TV_SCORE_AUTO && mode != TV_SCORE_L_CLASSIC && mode != TV_SCORE_L_U32 && mode != TV_SCORE_P)
+        return TV_ERR_BAD_ARGUMENT;
+    if (mode == TV_SCORE_P && ix->geo.bits != 4) { g_last_error = "score mode P needs 4-bit codes"; return TV_ERR_BAD_ARGUMENT; }
+    ix->score_mode = mode;
+    return TV_OK;
+}
+
+int tv_index_get_tables(const tv_index *ix, float *signs, uint32_t *perms, float *centroids, float *boundaries) {
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    if (signs) std::memcpy(signs, ix->rot.signs.data(), ix->rot.signs.size() * sizeof(float));
+    if (perms) std::memcpy(perms, ix->rot.perms.data(), ix->rot.perms.size() * sizeof(uint32_t));
+    if (centroids) std::memcpy(centroids, ix->cb.centroids.data(), ix->cb.centroids.size() * sizeof(float));
+    if (boundaries) std::memcpy(boundaries, ix->cb.boundaries.data(), ix->cb.boundaries.size() * sizeof(float));
+    return TV_OK;
+}
+
+int tv_index_upload_seq(tv_index *ix, const uint8_t *seq_codes, size_t n_vectors, const float *scales) {
+    if (!ix || (n_vectors && (!seq_codes || !scales))) return TV_ERR_BAD_ARGUMENT;
+    if (n_vectors >= (size_t(1) << 31)) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    ix->n = 0;
+    int rc = ensure_capacity(ix, n_vectors);
+    if (rc != TV_OK) return rc;
+    const tv::Geometry &g = ix->geo;
+    const size_t n_blocks = (n_vectors + tv::kVecBlock - 1) / tv::kVecBlock;
+    const size_t seq_block = size_t(g.G) * tv::kVecBlock;
+    // stage the sequential-blocked bytes through the workspace in slices
+    const size_t slice_blocks = std::max<size_t>(1, (size_t(256) << 20) / seq_block);
+    rc = ensure_workspace(ix, std::min(n_blocks, slice_blocks) * seq_block + 256);
+    if (rc != TV_OK) return rc;
+    for (size_t b0 = 0; b0 < n_blocks; b0 += slice_blocks) {
+        const size_t nb = std::min(slice_blocks, n_blocks - b0);
+        TV_HIP(hipMemcpyAsync(ix->ws, seq_codes + b0 * seq_block, nb * seq_block, hipMemcpyHostToDevice, ix->stream));
+        TV_HIP(tv::launch_seq_to_native(static_cast<const uint8_t *>(ix->ws), ix->d_codes, g, b0, nb, ix->stream));
+        TV_HIP(hipStreamSynchronize(ix->stream));
+    }
+    if (n_vectors) {
+        TV_HIP(hipMemsetAsync(ix->d_scales, 0, n_blocks * tv::kVecBlock * sizeof(float), ix->stream));
+        TV_HIP(hipMemcpyAsync(ix->d_scales, scales, n_vectors * sizeof(float), hipMemcpyHostToDevice, ix->stream));
+        TV_HIP(hipStreamSynchronize(ix->stream));
+    }
+    ix->n = n_vectors;
+    return TV_OK;
+}
+
+int tv_index_append_rows(tv_index *ix, const uint8_t *rows, const float *scales, size_t n_new) {
+    if (!ix || (n_new && (!rows || !scales))) return TV_ERR_BAD_ARGUMENT;
+    if (n_new == 0) return TV_OK;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    if (ix->n + n_new >= (size_t(1) << 31)) return TV_ERR_BAD_ARGUMENT;
+    int rc = ensure_capacity(ix, ix->n + n_new);
+    if (rc != TV_OK) return rc;
+    const tv::Geometry &g = ix->geo;
+    const size_t slice = std::max<size_t>(1, (size_t(64) << 20) / size_t(g.G));
+    rc = ensure_workspace(ix, std::min(n_new, slice) * size_t(g.G) + 256);
+    if (rc != TV_OK) return rc;
+    for (size_t r0 = 0; r0 < n_new; r0 += slice) {
+        const size_t nr = std::min(slice, n_new - r0);
+        TV_HIP(hipMemcpyAsync(ix->ws, rows + r0 * g.G, nr * size_t(g.G), hipMemcpyHostToDevice, ix->stream));
+        TV_HIP(tv::launch_append_rows(static_cast<const uint8_t *>(ix->ws), ix->d_codes, g, ix->n + r0, nr, ix->stream));
+        TV_HIP(hipStreamSynchronize(ix->stream));
+    }
+    TV_HIP(hipMemcpyAsync(ix->d_scales + ix->n, scales, n_new * sizeof(float), hipMemcpyHostToDevice, ix->stream));
+    TV_HIP(hipStreamSynchronize(ix->stream));
+    ix->n += n_new;
+    return TV_OK;
+}
+
+int tv_index_swap_remove(tv_index *ix, size_t idx) {
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    if (idx >= ix->n) return TV_ERR_INDEX_OUT_OF_RANGE;
+    TV_HIP(hipSetDevice(ix->device));
+    TV_HIP(tv::launch_move_lane(ix->d_codes, ix->d_scales, ix->geo, ix->n - 1, idx, ix->stream));
+    TV_HIP(hipStreamSynchronize(ix->stream));
+    ix->n -= 1;
+    return TV_OK;
+}
+
+int tv_index_download_seq(const tv_index *cix, uint8_t *seq_out, float *scales_out) {
+    tv_index *ix = const_cast<tv_index *>(cix);
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    const tv::Geometry &g = ix->geo;
+    const size_t n_blocks = (ix->n + tv::kVecBlock - 1) / tv::kVecBlock;
+    const size_t seq_block = size_t(g.G) * tv::kVecBlock;
+    if (seq_out && n_blocks) {
+        const size_t slice_blocks = std::max<size_t>(1, (size_t(256) << 20) / seq_block);
+        int rc = ensure_workspace(ix, std::min(n_blocks, slice_blocks) * seq_block + 256);
+        if (rc != TV_OK) return rc;
+        for (size_t b0 = 0; b0 < n_blocks; b0 += slice_blocks) {
+            const size_t nb = std::min(slice_blocks, n_blocks - b0);
+            TV_HIP(tv::launch_native_to_seq(ix->d_codes, static_cast<uint8_t *>(ix->ws), g, b0, nb, ix->stream));
+            TV_HIP(hipMemcpyAsync(seq_out + b0 * seq_block, ix->ws, nb * seq_block, hipMemcpyDeviceToHost, ix->stream));
+            TV_HIP(hipStreamSynchronize(ix->stream));
+        }
+    }
+    if (scales_out && ix->n) {
+        TV_HIP(hipMemcpyAsync(scales_out, ix->d_scales, ix->n * sizeof(float), hipMemcpyDeviceToHost, ix->stream));
+        TV_HIP(hipStreamSynchronize(ix->stream));
+    }
+    return TV_OK;
+}
+
+size_t tv_index_len(const tv_index *ix) { return ix ? ix->n : 0; }
+int tv_index_dim(const tv_index *ix) { return ix ? ix->geo.dim : 0; }
+int tv_index_bits(const tv_index *ix) { return ix ? ix->geo.bits : 0; }
+
+int tv_validate_queries(const float *queries, size_t len, int dim, size_t *bad_index) {
+    if (dim <= 0 || len % size_t(dim) != 0) return TV_ERR_QUERY_BUFFER_NOT_MULTIPLE_OF_DIM;
+    for (size_t i = 0; i < len; ++i) {
+        if (!(std::fabs(queries[i]) < 1e16f)) {
+            if (bad_index) *bad_index = i;
+            return TV_ERR_INVALID_QUERY_VALUE;
+        }
+    }
+    return TV_OK;
+}
+
+int tv_pack_mask(const uint8_t *mask_bytes, size_t n, uint64_t *words_out, size_t *n_allowed) {
+    if ((n && !mask_bytes) || !words_out) return TV_ERR_BAD_ARGUMENT;
+    size_t allowed = 0;
+    for (size_t w = 0; w * 64 < n; ++w) {
+        uint64_t word = 0;
+        const size_t lim = std::min<size_t>(64, n - w * 64);
+        for (size_t bit = 0; bit < lim; ++bit) word |= uint64_t(mask_bytes[w * 64 + bit] != 0) << bit;
+        allowed += size_t(__builtin_popcountll(word));
+        words_out[w] = word;
+    }
+    if (n_allowed) *n_allowed = allowed;
+    return TV_OK;
+}
+
+int tv_search_dev(tv_index *ix, const float *d_queries, size_t nq, size_t k, const uint64_t *d_mask_words,
+                  size_t n_allowed, float *d_out_scores, int64_t *d_out_indices, size_t *out_k_eff) {
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    if (!d_mask_words) n_allowed = ix->n;
+    return search_device(ix, d_queries, nq, k, d_mask_words, n_allowed, d_out_scores, d_out_indices, out_k_eff);
+}
+
+int tv_search(tv_index *ix, const float *queries, size_t nq, size_t k, const uint64_t *mask_words,
+              size_t n_mask_words, float *out_scores, int64_t *out_indices, size_t *out_k_eff) {
+    if (!ix || (nq && !queries)) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    const size_t n = ix->n;
+    size_t n_allowed = n;
+    if (mask_words) {
+        if (n_mask_words != (n + 63) / 64) return TV_ERR_MASK_LENGTH_MISMATCH;
+        n_allowed = 0;  // search.rs:3222-3225; bits at or past n are ignored
+        for (size_t w = 0; w < n_mask_words; ++w) {
+            uint64_t word = mask_words[w];
+            if (w * 64 + 64 > n) word &= (n - w * 64 >= 64) ? ~uint64_t(0) : ((uint64_t(1) << (n - w * 64)) - 1);
+            n_allowed += size_t(__builtin_popcountll(word));
+        }
+    }
+    const size_t k_eff = std::min(std::min(k, n), n_allowed);
+    if (out_k_eff) *out_k_eff = k_eff;
+    ix->last_scan_ms = 0.0f;
+    ix->last_scan_launches = 0;
+    if (k_eff == 0 || nq == 0) return TV_OK;
+    // host staging: queries, mask and results live in their own allocations so
+    // the per-chunk workspace can be re-carved freely
+    const size_t dim = size_t(ix->geo.dim);
+    float *d_q = nullptr, *d_s = nullptr;
+    int64_t *d_i = nullptr;
+    uint64_t *d_m = nullptr;
+    int rc = TV_OK;
+    do {
+        if (hipMalloc(reinterpret_cast<void **>(&d_q), nq * dim * sizeof(float)) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void **>(&d_s), nq * k_eff * sizeof(float)) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void **>(&d_i), nq * k_eff * sizeof(int64_t)) != hipSuccess ||
+            (mask_words && hipMalloc(reinterpret_cast<void **>(&d_m), n_mask_words * 8) != hipSuccess)) {
+            g_last_error = "device allocation failed";
+            rc = TV_ERR_HIP;
+            break;
+        }
+        if (hipMemcpyAsync(d_q, queries, nq * dim * sizeof(float), hipMemcpyHostToDevice, ix->stream) != hipSuccess ||
+            (mask_words && hipMemcpyAsync(d_m, mask_words, n_mask_words * 8, hipMemcpyHostToDevice, ix->stream) != hipSuccess)) {
+            g_last_error = "host to device copy failed";
+            rc = TV_ERR_HIP;
+            break;
+        }
+        rc = search_device(ix, d_q, nq, k, d_m, n_allowed, d_s, d_i, nullptr);
+        if (rc != TV_OK) break;
+        if (hipMemcpyAsync(out_scores, d_s, nq * k_eff * sizeof(float), hipMemcpyDeviceToHost, ix->stream) != hipSuccess ||
+            hipMemcpyAsync(out_indices, d_i, nq * k_eff * sizeof(int64_t), hipMemcpyDeviceToHost, ix->stream) != hipSuccess ||
+            hipStreamSynchronize(ix->stream) != hipSuccess) {
+            g_last_error = "device to host copy failed";
+            rc = TV_ERR_HIP;
+        }
+    } while (0);
+    if (d_q) (void)hipFree(d_q);
+    if (d_s) (void)hipFree(d_s);
+    if (d_i) (void)hipFree(d_i);
+    if (d_m) (void)hipFree(d_m);
+    return rc;
+}
+
+int tv_debug_scan(tv_index *ix, const float *queries, size_t nq, int32_t *acc_out, float *scores_out) {
+    if (!ix || (nq && !queries)) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    const size_t n = ix->n;
+    if (n == 0 || nq == 0) return TV_OK;
+    const tv::Geometry &g = ix->geo;
+    const int mode = effective_mode(ix);
+    const bool mode_p = mode == TV_SCORE_P;
+    const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_tile_queries(g.nch, 1));
+    for (size_t q0 = 0; q0 < nq; q0 += tile_q) {
+        const size_t cq = std::min<size_t>(tile_q, nq - q0);
+        size_t need = prepare_bytes(ix, cq) + round_up(cq * g.dim * 4, 256) + 2 * round_up(cq * n * 4, 256) + 65536;
+        int rc = ensure_workspace(ix, need);
+        if (rc != TV_OK) return rc;
+        Arena ar;
+        ar.base = static_cast<uint8_t *>(ix->ws);
+        float *d_q = ar.take<float>(cq * g.dim);
+        int32_t *d_acc = ar.take<int32_t>(cq * n);
+        float *d_sc = ar.take<float>(cq * n);
+        TV_HIP(hipMemcpyAsync(d_q, queries + q0 * g.dim, cq * g.dim * sizeof(float), hipMemcpyHostToDevice, ix->stream));
+        Prepared pq;
+        rc = prepare_queries(ix, ar, d_q, cq, pq);
+        if (rc != TV_OK) return rc;
+        tv::ScanArgs a;
+        fill_scan_args(ix, a);
+        a.tables = pq.d_tables;
+        a.qscale = pq.d_qscale;
+        a.qbias = pq.d_qbias;
+        a.nq_tile = int(cq);
+        a.k = 1;
+        a.acc_out = d_acc;
+        a.score_out = d_sc;
+        const int grid = tv::scan_grid_blocks(ix->device, mode_p, g.nch, 1, int(tile_q));
+        if (mode_p) TV_HIP(tv::launch_scan_p4(a, grid, true, ix->stream));
+        else TV_HIP(tv::launch_scan_lut(a, grid, true, ix->stream));
+        if (acc_out) TV_HIP(hipMemcpyAsync(acc_out + q0 * n, d_acc, cq * n * 4, hipMemcpyDeviceToHost, ix->stream));
+        if (scores_out) TV_HIP(hipMemcpyAsync(scores_out + q0 * n, d_sc, cq * n * 4, hipMemcpyDeviceToHost, ix->stream));
+        TV_HIP(hipStreamSynchronize(ix->stream));
+    }
+    return TV_OK;
+}
+
+int tv_debug_prepare(tv_index *ix, const float *queries, size_t nq, float *q_rot_out, float *scale_out,
+                     float *bias_out) {
+    if (!ix || (nq && !queries)) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    if (nq == 0) return TV_OK;
+    const tv::Geometry &g = ix->geo;
+    int rc = ensure_workspace(ix, prepare_bytes(ix, nq) + round_up(nq * g.dim * 4, 256) + 65536);
+    if (rc != TV_OK) return rc;
+    Arena ar;
+    ar.base = static_cast<uint8_t *>(ix->ws);
+    float *d_q = ar.take<float>(nq * g.dim);
+    TV_HIP(hipMemcpyAsync(d_q, queries, nq * g.dim * sizeof(float), hipMemcpyHostToDevice, ix->stream));
+    Prepared pq;
+    rc = prepare_queries(ix, ar, d_q, nq, pq);
+    if (rc != TV_OK) return rc;
+    if (q_rot_out) TV_HIP(hipMemcpyAsync(q_rot_out, pq.d_qrot, nq * g.dim * 4, hipMemcpyDeviceToHost, ix->stream));
+    if (scale_out) TV_HIP(hipMemcpyAsync(scale_out, pq.d_qscale, nq * 4, hipMemcpyDeviceToHost, ix->stream));
+    if (bias_out) TV_HIP(hipMemcpyAsync(bias_out, pq.d_qbias, nq * 4, hipMemcpyDeviceToHost, ix->stream));
+    TV_HIP(hipStreamSynchronize(ix->stream));
+    return TV_OK;
+}
+
+int tv_last_scan_ms(const tv_index *ix, float *ms, int *launches) {
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    if (ms) *ms = ix->last_scan_ms;
+    if (launches) *launches = ix->last_scan_launches;
+    return TV_OK;
+}
+
+int tv_index_device_ptrs(const tv_index *ix, void **d_codes, void **d_scales, size_t *code_bytes) {
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    if (d_codes) *d_codes = ix->d_codes;
+    if (d_scales) *d_scales = ix->d_scales;
+    if (code_bytes) *code_bytes = (ix->n + tv::kVecBlock - 1) / tv::kVecBlock * ix->geo.block_bytes();
+    return TV_OK;
+}
+
+}  // extern "C"

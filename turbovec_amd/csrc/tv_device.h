@@ -1,0 +1,87 @@
+// Device-side helpers shared by the scan, merge and select kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace tv {
+
+// ===========================================================================
+// Top-k bookkeeping shared by the scan kernels and the merge kernel.
+// Total order: higher score first, ties to the lower slot
+// (turbovec/src/search.rs:244-252 and :4285-4289).  Float compares make
+// -0.0 and +0.0 tie, as partial_cmp does.
+// ===========================================================================
+
+__device__ __forceinline__ bool ranks_before(float s, uint32_t i, float s2, uint32_t i2) {
+    return s > s2 || (s == s2 && i < i2);
+}
+
+// Monotone float -> signed int key (for atomicMax on thresholds).
+__device__ __forceinline__ int order_key(float f) {
+    const int b = __float_as_int(f);
+    return b ^ ((b >> 31) & 0x7fffffff);
+}
+__device__ __forceinline__ float order_unkey(int k) { return __int_as_float(k ^ ((k >> 31) & 0x7fffffff)); }
+// order_key(-infinity): the threshold every real score passes.
+constexpr int kTauInit = int(0x807fffffu);
+
+// A lane-private unsorted list of up to k entries living in LDS at
+// ls/li[entry * stride + slot_of_lane]; the lane keeps its size, and its worst
+// entry (score, index, position) in registers.
+struct LaneList {
+    int cnt;
+    float worst_s;
+    uint32_t worst_i;
+    int worst_pos;
+};
+
+__device__ __forceinline__ void list_rescan(LaneList &L, const float *ls, const uint32_t *li, int stride, int me,
+                                            int k) {
+    float ws = ls[me];
+    uint32_t wi = li[me];
+    int wp = 0;
+    for (int e = 1; e < k; ++e) {
+        const float s = ls[e * stride + me];
+        const uint32_t i = li[e * stride + me];
+        if (ranks_before(ws, wi, s, i)) { ws = s; wi = i; wp = e; }
+    }
+    L.worst_s = ws; L.worst_i = wi; L.worst_pos = wp;
+}
+
+// Returns true when the list is full after the call and its worst entry changed.
+__device__ __forceinline__ bool list_offer(LaneList &L, float *ls, uint32_t *li, int stride, int me, int k, float s,
+                                           uint32_t idx) {
+    if (L.cnt < k) {
+        ls[L.cnt * stride + me] = s;
+        li[L.cnt * stride + me] = idx;
+        ++L.cnt;
+        if (L.cnt == k) { list_rescan(L, ls, li, stride, me, k); return true; }
+        return false;
+    }
+    if (!ranks_before(s, idx, L.worst_s, L.worst_i)) return false;
+    ls[L.worst_pos * stride + me] = s;
+    li[L.worst_pos * stride + me] = idx;
+    list_rescan(L, ls, li, stride, me, k);
+    return true;
+}
+
+__device__ __forceinline__ uint64_t sort_key(float s, uint32_t idx) {
+    // high word: order key of the score with -0.0 folded onto +0.0 (they tie);
+    // low word: inverted slot so that the lower slot sorts first, plus one bit
+    // remembering a negative zero so the emitted score keeps its sign bit.
+    const bool negzero = __float_as_uint(s) == 0x80000000u;
+    const float canon = negzero ? 0.0f : s;
+    const uint32_t hi = uint32_t(order_key(canon)) ^ 0x80000000u;
+    const uint32_t lo = ((0x7fffffffu - idx) << 1) | (negzero ? 1u : 0u);
+    return (uint64_t(hi) << 32) | lo;
+}
+__device__ __forceinline__ void sort_unkey(uint64_t key, float &s, uint32_t &idx) {
+    const uint32_t hi = uint32_t(key >> 32), lo = uint32_t(key);
+    s = order_unkey(int(hi ^ 0x80000000u));
+    if (lo & 1u) s = -0.0f;
+    idx = 0x7fffffffu - (lo >> 1);
+}
+
+
+}  // namespace tv

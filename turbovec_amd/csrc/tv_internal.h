@@ -1,0 +1,124 @@
+// Internal declarations shared by the HIP kernels and the C-ABI host code.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <mutex>
+#include <vector>
+
+#include "host_tables.h"
+
+namespace tv {
+
+constexpr int kVecBlock = 32;    // vectors per block (turbovec/src/lib.rs:89)
+constexpr int kChunkGroups = 32; // byte-groups per native chunk
+constexpr int kQTile = 32;       // queries per MFMA column tile
+constexpr int kScanThreads = 256;
+constexpr int kMaxListK = 32;    // largest k served by the per-lane lists
+
+// Native device layout of the codes ("vm32"): the byte of (block b, group g,
+// vector i) lives at ((b*nch + g/32)*64 + ((g%32)/16)*32 + i)*16 + g%16, groups
+// padded with zero bytes to a multiple of 32.  One 64-lane wave reads a chunk
+// (32 vectors x 32 groups = 1 KiB) with one 16-byte load per lane, and the 16
+// bytes a lane receives are 16 consecutive groups of ONE vector -- the operand
+// shape of the i8 MFMA and of the per-vector LUT walk alike.
+struct Geometry {
+    int dim = 0, bits = 0;
+    int G = 0;    // byte groups per vector = dim*bits/8 (3-bit: dim/2)
+    int nch = 0;  // chunks per block = ceil(G/32)
+    size_t block_bytes() const { return size_t(nch) * 1024; }
+};
+
+struct ScanArgs {
+    const uint8_t *codes;
+    const float *scales;       // padded to a multiple of 32 entries
+    const uint64_t *mask;      // nullptr = unfiltered
+    const uint8_t *tables;     // this tile's weight fragments (mode P) or LUTs (mode L)
+    const float *qscale;       // this tile's per-query scale (kQTile entries)
+    const float *qbias;
+    int nq_tile;
+    uint32_t n;
+    uint32_t n_blocks;
+    int nch;
+    int k;
+    uint32_t lv[4];            // the 16 int8 codebook levels, little-endian packed
+    int *gtau;                 // kQTile running thresholds (orderable ints)
+    float *part_scores;        // [k][total_threads]
+    uint32_t *part_idx;
+    int *part_cnt;             // [total_threads]
+    int32_t *acc_out;          // dump mode: [nq_tile][n] (may be null)
+    float *score_out;          // dump mode: [nq_tile][n]
+    int classic;               // mode L: 1 = fma flush per 256 groups, 0 = u32 epilogue
+};
+
+// ---- launchers (tv_kernels.hip) ----
+hipError_t launch_seq_to_native(const uint8_t *d_seq, uint8_t *d_native, const Geometry &g, size_t first_block,
+                                size_t n_blocks, hipStream_t s);
+hipError_t launch_native_to_seq(const uint8_t *d_native, uint8_t *d_seq, const Geometry &g, size_t first_block,
+                                size_t n_blocks, hipStream_t s);
+hipError_t launch_append_rows(const uint8_t *d_rows, uint8_t *d_native, const Geometry &g, size_t old_n,
+                              size_t n_new, hipStream_t s);
+hipError_t launch_move_lane(uint8_t *d_native, float *d_scales, const Geometry &g, size_t src, size_t dst,
+                            hipStream_t s);
+
+hipError_t launch_rotate(const float *d_q, float *d_out, const float *d_signs, const uint32_t *d_perms, int dim,
+                         int block, float inv_sqrt_block, size_t nq, hipStream_t s);
+hipError_t launch_calibrate(const float *d_qrot, float *d_qcal, float *d_bias_corr, const float *d_shift,
+                            const float *d_scale, int dim, size_t nq, hipStream_t s);
+hipError_t launch_build_p(const float *d_qcal, const float *d_bias_corr, uint8_t *d_wfrag, float *d_qscale,
+                          float *d_qbias, int dim, int G, int nch, float cs, size_t nq, size_t nq_padded,
+                          hipStream_t s);
+hipError_t launch_build_lut(const float *d_qcal, const float *d_bias_corr, const float *d_centroids, uint8_t *d_lut,
+                            float *d_qscale, float *d_qbias, int dim, int bits, int G, int nch, size_t nq,
+                            size_t nq_padded, hipStream_t s);
+
+int scan_grid_blocks(int device, int mode_p, int nch, int k, int lut_queries);
+size_t scan_lds_bytes(int mode_p, int nch, int k, int lut_queries);
+// Queries one launch of the LUT scan serves (1, 2 or 4), from the LDS budget.
+int lut_tile_queries(int nch, int k);
+// Queries per LDS entry (1, 2 or 4) the LUT scan launch picks for nq_tile queries.
+int lut_launch_ql(int nch, int k, int nq_tile);
+hipError_t launch_scan_p4(const ScanArgs &a, int grid, bool dump, hipStream_t s);
+hipError_t launch_scan_lut(const ScanArgs &a, int grid, bool dump, hipStream_t s);
+hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, const int *part_cnt, int total_threads,
+                        int qmod, int k, int k_eff, int nq_tile, float *out_scores, int64_t *out_idx,
+                        hipStream_t s);
+hipError_t launch_fill_i32(int *p, int v, size_t n, hipStream_t s);
+// Exact top-k of a dense score row per query (NaN = excluded slot).
+hipError_t launch_select_topk(const float *d_scores, size_t n, int nq_tile, size_t k_eff, uint64_t *d_keys_tmp,
+                              uint32_t *d_hist, float *out_scores, int64_t *out_idx, hipStream_t s);
+size_t select_tmp_keys(size_t k_eff);
+
+}  // namespace tv
+
+// The opaque handle of the C ABI.
+struct tv_index {
+    tv::Geometry geo;
+    int device = 0;
+    int score_mode = 0;
+    tv::RotationTables rot;
+    tv::Codebook cb;
+    std::vector<float> tq_shift, tq_scale;
+    int8_t levels[16] = {0};
+    float cs = 1.0f;
+
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    float *d_signs = nullptr;
+    uint32_t *d_perms = nullptr;
+    float *d_centroids = nullptr;
+    float *d_tq_shift = nullptr, *d_tq_scale = nullptr;
+
+    uint8_t *d_codes = nullptr;
+    float *d_scales = nullptr;
+    size_t cap_blocks = 0;
+    size_t n = 0;
+
+    // per-search workspace, grown on demand, guarded by mu
+    mutable std::mutex mu;
+    void *ws = nullptr;
+    size_t ws_bytes = 0;
+    float last_scan_ms = 0.0f;
+    int last_scan_launches = 0;
+};

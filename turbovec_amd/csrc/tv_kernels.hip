@@ -1,0 +1,681 @@
+// HIP kernels of the turbovec search path for gfx950 (MI355X).
+//
+// Compiled with -ffp-contract=off: every float expression keeps the separate
+// multiplies and adds the reference performs, and fmaf appears only where the
+// reference fuses.
+#include "tv_internal.h"
+#include "tv_device.h"
+
+#include <cfloat>
+#include <climits>
+
+namespace tv {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// ===========================================================================
+// Layout transforms between the persisted sequential-blocked layout
+// (turbovec/src/pack.rs:336-361) and the native chunked layout.
+// ===========================================================================
+
+// One workgroup per (block, chunk): a 1 KiB tile of 32 groups x 32 lanes is
+// transposed through LDS so both sides move as dwords.
+__global__ __launch_bounds__(256) void k_seq_to_native(const uint8_t *__restrict__ seq, uint8_t *__restrict__ nat,
+                                                       int G, int nch, size_t first_block) {
+    __shared__ uint8_t tile[32 * 36];  // [group][lane], rows padded to 36 bytes
+    const size_t b = first_block + blockIdx.x / nch;
+    const int c = blockIdx.x % nch;
+    const int t = threadIdx.x;
+    {   // read: dword t covers group gl = t/8, lanes 4*(t%8)..+3
+        const int gl = t >> 3, l4 = (t & 7) * 4;
+        const int g = c * 32 + gl;
+        uint32_t v = 0;
+        if (g < G) v = *reinterpret_cast<const uint32_t *>(seq + ((b - first_block) * size_t(G) + g) * 32 + l4);
+        *reinterpret_cast<uint32_t *>(tile + gl * 36 + l4) = v;
+    }
+    __syncthreads();
+    {   // write: dword t of the chunk = lane l = t/4 (h = l/32, i = l%32), bytes j0..j0+3
+        const int l = t >> 2, j0 = (t & 3) * 4;
+        const int h = l >> 5, i = l & 31;
+        uint32_t v = 0;
+        for (int j = 0; j < 4; ++j) v |= uint32_t(tile[(16 * h + j0 + j) * 36 + i]) << (8 * j);
+        *reinterpret_cast<uint32_t *>(nat + (b * size_t(nch) + c) * 1024 + size_t(t) * 4) = v;
+    }
+}
+
+__global__ __launch_bounds__(256) void k_native_to_seq(const uint8_t *__restrict__ nat, uint8_t *__restrict__ seq,
+                                                       int G, int nch, size_t first_block) {
+    __shared__ uint8_t tile[32 * 36];
+    const size_t b = first_block + blockIdx.x / nch;
+    const int c = blockIdx.x % nch;
+    const int t = threadIdx.x;
+    {
+        const int l = t >> 2, j0 = (t & 3) * 4;
+        const int h = l >> 5, i = l & 31;
+        const uint32_t v = *reinterpret_cast<const uint32_t *>(nat + (b * size_t(nch) + c) * 1024 + size_t(t) * 4);
+        for (int j = 0; j < 4; ++j) tile[(16 * h + j0 + j) * 36 + i] = uint8_t(v >> (8 * j));
+    }
+    __syncthreads();
+    {
+        const int gl = t >> 3, l4 = (t & 7) * 4;
+        const int g = c * 32 + gl;
+        if (g < G)
+            *reinterpret_cast<uint32_t *>(seq + ((b - first_block) * size_t(G) + g) * 32 + l4) =
+                *reinterpret_cast<const uint32_t *>(tile + gl * 36 + l4);
+    }
+}
+
+__device__ __forceinline__ size_t native_byte_index(size_t v, int g, int nch) {
+    const size_t b = v >> 5;
+    const int i = int(v & 31);
+    return ((b * size_t(nch) + size_t(g >> 5)) * 64 + size_t(((g & 31) >> 4) * 32 + i)) * 16 + size_t(g & 15);
+}
+
+// rows[r*G + g] -> lane of vector old_n + r (turbovec/src/pack.rs:211-233 append_lanes).
+__global__ void k_append_rows(const uint8_t *__restrict__ rows, uint8_t *__restrict__ nat, int G, int nch,
+                              size_t old_n, size_t n_new) {
+    const size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= n_new * size_t(G)) return;
+    const size_t r = idx / G;
+    const int g = int(idx % G);
+    nat[native_byte_index(old_n + r, g, nch)] = rows[idx];
+}
+
+// turbovec/src/lib.rs:2964-3003: move_lane(last -> idx), zero_lane(last), scale move.
+__global__ void k_move_lane(uint8_t *__restrict__ nat, float *__restrict__ scales, int G, int nch, size_t src,
+                            size_t dst) {
+    const int g = blockIdx.x * blockDim.x + threadIdx.x;
+    if (g < G) {
+        const size_t s = native_byte_index(src, g, nch);
+        if (src != dst) nat[native_byte_index(dst, g, nch)] = nat[s];
+        nat[s] = 0;
+    }
+    if (g == 0) {
+        if (src != dst) scales[dst] = scales[src];
+        scales[src] = 0.0f;
+    }
+}
+
+__global__ void k_fill_i32(int *p, int v, size_t n) {
+    const size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// ===========================================================================
+// Query preparation
+// ===========================================================================
+
+// turbovec/src/rotation.rs:265-320 (apply_with_scratch) + :964-982 (wht_block_scalar).
+// One workgroup per query row; both rounds run in LDS.  Every output element is
+// produced by the same IEEE adds, subtracts and multiplies, in the same
+// operand pairing, as the scalar butterfly, so the result is bit-identical.
+__global__ __launch_bounds__(256) void k_rotate(const float *__restrict__ q, float *__restrict__ out,
+                                                const float *__restrict__ signs,
+                                                const uint32_t *__restrict__ perms, int dim, int block,
+                                                float inv_sqrt_block) {
+    extern __shared__ float rot_lds[];
+    float *A = rot_lds;
+    float *B = rot_lds + dim;
+    const float *src = q + size_t(blockIdx.x) * dim;
+    const int t = threadIdx.x;
+    for (int i = t; i < dim; i += 256) A[i] = src[perms[i]] * signs[i];
+    __syncthreads();
+    for (int len = 1; len < block; len <<= 1) {
+        for (int p = t; p < dim / 2; p += 256) {
+            const int j = 2 * p - (p & (len - 1));
+            const float a = A[j], b = A[j + len];
+            A[j] = a + b;
+            A[j + len] = a - b;
+        }
+        __syncthreads();
+    }
+    // the 1/sqrt(B) scale of round 0 rides the round-1 gather: (x * inv) * sign
+    for (int i = t; i < dim; i += 256) B[i] = (A[perms[dim + i]] * inv_sqrt_block) * signs[dim + i];
+    __syncthreads();
+    for (int len = 1; len < block; len <<= 1) {
+        for (int p = t; p < dim / 2; p += 256) {
+            const int j = 2 * p - (p & (len - 1));
+            const float a = B[j], b = B[j + len];
+            B[j] = a + b;
+            B[j + len] = a - b;
+        }
+        __syncthreads();
+    }
+    float *dst = out + size_t(blockIdx.x) * dim;
+    for (int i = t; i < dim; i += 256) dst[i] = B[i] * inv_sqrt_block;
+}
+
+// turbovec/src/search.rs:3154-3186 calibrate_queries.  The f64 bias sum is
+// sequential over d, so one thread carries it.
+__global__ __launch_bounds__(256) void k_calibrate(const float *__restrict__ qrot, float *__restrict__ qcal,
+                                                   float *__restrict__ bias_corr,
+                                                   const float *__restrict__ shift,
+                                                   const float *__restrict__ scale, int dim) {
+    const float *src = qrot + size_t(blockIdx.x) * dim;
+    float *dst = qcal + size_t(blockIdx.x) * dim;
+    for (int i = threadIdx.x; i < dim; i += 256) dst[i] = src[i] / scale[i];
+    if (threadIdx.x == 0) {
+        double bc = 0.0;
+        for (int d = 0; d < dim; ++d) bc -= double(src[d]) * double(shift[d]);
+        bias_corr[blockIdx.x] = float(bc);
+    }
+}
+
+__device__ __forceinline__ float block_max_256(float v, float *red) {
+    // exact: max is order-free
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    v = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    return v;
+}
+
+__device__ __forceinline__ float clamp_round_i8(float v) {
+    // Rust f32::round is half-away-from-zero, like roundf; then clamp(-127, 127)
+    v = roundf(v);
+    return v < -127.0f ? -127.0f : (v > 127.0f ? 127.0f : v);
+}
+
+// turbovec/src/search.rs:2806-2846 build_permute_dot, emitting the weights in
+// the MFMA B-fragment order of the scan: for query tile t, chunk c and nibble
+// plane p (0 = low nibble = odd dimension, 1 = high nibble = even dimension) a
+// 1 KiB fragment whose lane (h*32 + n) holds the 16 weights of query n for
+// groups 32c + 16h .. +15.
+__global__ __launch_bounds__(256) void k_build_p(const float *__restrict__ qcal,
+                                                 const float *__restrict__ bias_corr,
+                                                 uint8_t *__restrict__ wfrag, float *__restrict__ qscale,
+                                                 float *__restrict__ qbias, int dim, int G, int nch, float cs,
+                                                 size_t nq) {
+    __shared__ float red[4];
+    const size_t qi = blockIdx.x;
+    const size_t tile = qi / kQTile;
+    const int n = int(qi % kQTile);
+    uint8_t *base = wfrag + tile * size_t(nch) * 2048;
+    const int t = threadIdx.x;
+    if (qi >= nq) {  // padding query of the last tile: zero weights
+        for (int g = t; g < nch * 32; g += 256) {
+            const size_t off = size_t(g >> 5) * 2048 + size_t(((g & 31) >> 4) * 32 + n) * 16 + size_t(g & 15);
+            base[off] = 0;
+            base[off + 1024] = 0;
+        }
+        if (t == 0) { qscale[qi] = 0.0f; qbias[qi] = 0.0f; }
+        return;
+    }
+    const float *q = qcal + qi * size_t(dim);
+    float m = 0.0f;
+    for (int d = t; d < dim; d += 256) m = fmaxf(m, fabsf(q[d]));
+    const float qmax = block_max_256(m, red);
+    float qs = qmax / 127.0f, inv_qs;
+    if (qs >= FLT_MIN) inv_qs = 1.0f / qs; else { qs = 1.0f; inv_qs = 1.0f; }
+    for (int g = t; g < nch * 32; g += 256) {
+        int8_t lo = 0, hi = 0;
+        if (g < G) {
+            lo = int8_t(clamp_round_i8(q[2 * g + 1] * inv_qs));
+            hi = int8_t(clamp_round_i8(q[2 * g] * inv_qs));
+        }
+        const size_t off = size_t(g >> 5) * 2048 + size_t(((g & 31) >> 4) * 32 + n) * 16 + size_t(g & 15);
+        base[off] = uint8_t(lo);
+        base[off + 1024] = uint8_t(hi);
+    }
+    if (t == 0) {
+        qscale[qi] = cs * qs;
+        qbias[qi] = 0.0f + bias_corr[qi];
+    }
+}
+
+// turbovec/src/search.rs:2856-2994 build_query_neon_lut_from_slice.  Output per
+// query: nch*32 rows of 32 bytes, row g = [16 entries indexed by the byte's HIGH
+// nibble (the group's first dimensions) | 16 entries indexed by the LOW nibble];
+// rows of padding groups are zero.
+template <int BITS>
+__device__ __forceinline__ float lut_entry(const float *q, const float *cen, int dim_start, int sub, int nv) {
+    constexpr int cpb = 8 / BITS, cpn = cpb / 2;
+    constexpr unsigned code_mask = (1u << BITS) - 1;
+    float s = 0.0f;
+#pragma unroll
+    for (int c = 0; c < cpn; ++c) {
+        const int sh = (cpn - 1 - c) * BITS;
+        const unsigned code = (unsigned(nv) >> sh) & code_mask;
+        s += q[dim_start + sub * cpn + c] * cen[code];
+    }
+    return s;
+}
+
+template <int BITS>
+__global__ __launch_bounds__(256) void k_build_lut(const float *__restrict__ qcal,
+                                                   const float *__restrict__ bias_corr,
+                                                   const float *__restrict__ centroids,
+                                                   uint8_t *__restrict__ lut, float *__restrict__ qscale,
+                                                   float *__restrict__ qbias, int dim, int G, int nch, size_t nq) {
+    extern __shared__ float lut_lds[];  // mins: 2*G floats
+    __shared__ float red[4];
+    __shared__ float cen[16];
+    constexpr int cpb = 8 / BITS;
+    const size_t qi = blockIdx.x;
+    uint8_t *dst = lut + qi * size_t(nch) * 1024;
+    const int t = threadIdx.x;
+    if (qi >= nq) {
+        for (int i = t; i < nch * 256; i += 256) reinterpret_cast<uint32_t *>(dst)[i] = 0;
+        if (t == 0) { qscale[qi] = 0.0f; qbias[qi] = 0.0f; }
+        return;
+    }
+    if (t < (1 << BITS)) cen[t] = centroids[t];
+    __syncthreads();
+    const float *q = qcal + qi * size_t(dim);
+    float span = 0.0f;
+    for (int g = t; g < G; g += 256) {
+        for (int sub = 0; sub < 2; ++sub) {
+            float mn = FLT_MAX, mx = -FLT_MAX;
+            for (int nv = 0; nv < 16; ++nv) {
+                const float s = lut_entry<BITS>(q, cen, g * cpb, sub, nv);
+                if (s < mn) mn = s;
+                if (s > mx) mx = s;
+            }
+            lut_lds[2 * g + sub] = mn;
+            span = fmaxf(span, mx - mn);
+        }
+    }
+    const float max_span = block_max_256(span, red);  // also orders the lut_lds writes
+    float scale = max_span > 0.0f ? max_span / 127.0f : 1.0f, inv_scale;
+    if (scale >= FLT_MIN) inv_scale = 1.0f / scale; else { scale = 1.0f; inv_scale = 1.0f; }
+    if (t == 0) {
+        float bias = 0.0f;  // sequential f32 sum over groups, inner add first (search.rs:2910)
+        for (int g = 0; g < G; ++g) bias += lut_lds[2 * g] + lut_lds[2 * g + 1];
+        qscale[qi] = scale;
+        qbias[qi] = bias + bias_corr[qi];
+    }
+    for (int g = t; g < nch * 32; g += 256) {
+        uint32_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (g < G) {
+            for (int sub = 0; sub < 2; ++sub) {
+                const float mn = lut_lds[2 * g + sub];
+                for (int nv = 0; nv < 16; ++nv) {
+                    float v = roundf((lut_entry<BITS>(q, cen, g * cpb, sub, nv) - mn) * inv_scale);
+                    v = v < 0.0f ? 0.0f : (v > 127.0f ? 127.0f : v);
+                    w[sub * 4 + nv / 4] |= uint32_t(uint8_t(v)) << (8 * (nv & 3));
+                }
+            }
+        }
+        uint4 *o = reinterpret_cast<uint4 *>(dst + size_t(g) * 32);
+        o[0] = make_uint4(w[0], w[1], w[2], w[3]);
+        o[1] = make_uint4(w[4], w[5], w[6], w[7]);
+    }
+}
+
+// ===========================================================================
+// Scan, score mode P: 4-bit codes -> int8 codebook levels -> i8 MFMA against
+// int8 query weights (turbovec/src/search.rs:1392-1567 computes the same
+// integers with vpdpbusd).  acc = sum_d w[d] * level[code[d]], exact in i32;
+// score = fma(f32(acc), scale, bias) * vec_scale (search.rs:1519-1524).
+// ===========================================================================
+
+// Four packed nibbles (one per byte, values 0..15) -> four int8 levels.
+// v_perm_b32 looks up 8 table bytes; selectors >= 13 give 0xff, so each half
+// of the 16-entry table is looked up with the other half's nibbles pushed out
+// of range, and the two results are ANDed.
+__device__ __forceinline__ uint32_t levels_of(uint32_t nib, uint32_t t0, uint32_t t1, uint32_t t2, uint32_t t3) {
+    const uint32_t selA = nib + (nib & 0x08080808u);  // 0..7 stay, 8..15 -> 16..23
+    const uint32_t selB = selA ^ 0x10101010u;         // 0..7 -> 16..23, 16..23 -> 0..7
+    return __builtin_amdgcn_perm(t1, t0, selA) & __builtin_amdgcn_perm(t3, t2, selB);
+}
+
+template <int U, bool DUMP, bool W_LDS>
+__global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int nch = a.nch, k = a.k;
+    uint8_t *sW = smem;
+    const size_t w_bytes = W_LDS ? size_t(nch) * 2048 : 0;
+    float *ls = reinterpret_cast<float *>(smem + w_bytes);
+    uint32_t *li = reinterpret_cast<uint32_t *>(ls + (DUMP ? 0 : k * kScanThreads));
+    int *stau = reinterpret_cast<int *>(li + (DUMP ? 0 : k * kScanThreads));
+
+    const int tid = threadIdx.x;
+    if (W_LDS) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.tables);
+        uint4 *dst = reinterpret_cast<uint4 *>(sW);
+        for (int i = tid; i < nch * 128; i += kScanThreads) dst[i] = src[i];
+    }
+    if (!DUMP && tid < kQTile) stau[tid] = a.gtau[tid];
+    __syncthreads();
+
+    const int lane = tid & 63, wave = tid >> 6;
+    const int qn = lane & 31, h = lane >> 5;
+    const bool active = qn < a.nq_tile;
+    const float qs = active ? a.qscale[qn] : 0.0f;
+    const float qb = active ? a.qbias[qn] : 0.0f;
+    const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
+
+    const uint32_t total_waves = gridDim.x * (kScanThreads / 64);
+    const uint32_t gw = blockIdx.x * (kScanThreads / 64) + wave;
+    const uint32_t per = (a.n_blocks + total_waves - 1) / total_waves;
+    const uint32_t b_begin = min(gw * per, a.n_blocks);
+    const uint32_t b_end = min(b_begin + per, a.n_blocks);
+
+    LaneList L{0, 0.0f, 0u, 0};
+    const uint4 *codes = reinterpret_cast<const uint4 *>(a.codes) + lane;
+    const uint4 *wglob = reinterpret_cast<const uint4 *>(a.tables) + lane;
+    const uint4 *wlds = reinterpret_cast<const uint4 *>(sW) + lane;
+
+    // first block with at least one allowed slot (search.rs:3015-3029)
+    auto live_from = [&](uint32_t b) -> uint32_t {
+        if (a.mask == nullptr) return b;
+        while (b < b_end) {
+            const uint64_t w = a.mask[b >> 1];
+            if (uint32_t(w >> ((b & 1) * 32)) != 0u) break;
+            ++b;
+        }
+        return b;
+    };
+
+    uint32_t b = live_from(b_begin);
+    uint4 buf[U];
+    if (b < b_end) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(b) * nch + u) * 64];
+    }
+    while (b < b_end) {
+        const uint32_t nb = live_from(b + 1);
+        v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (int c0 = 0; c0 < nch; c0 += U) {
+            uint4 cur[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) cur[u] = buf[u];
+            if (c0 + U < nch) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(b) * nch + c0 + U + u) * 64];
+            } else if (nb < b_end) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(nb) * nch + u) * 64];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u;
+                const uint32_t x[4] = {cur[u].x, cur[u].y, cur[u].z, cur[u].w};
+                v4i alo, ahi;
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    alo[d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
+                    ahi[d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
+                }
+                uint4 wl, wh;
+                if (W_LDS) { wl = wlds[(c * 2) * 64]; wh = wlds[(c * 2 + 1) * 64]; }
+                else { wl = wglob[(size_t(c) * 2) * 64]; wh = wglob[(size_t(c) * 2 + 1) * 64]; }
+                const v4i blo = {int(wl.x), int(wl.y), int(wl.z), int(wl.w)};
+                const v4i bhi = {int(wh.x), int(wh.y), int(wh.z), int(wh.w)};
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo, blo, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi, bhi, acc, 0, 0, 0);
+            }
+        }
+
+        // ---- epilogue: lane owns query qn and rows 8*(r/4) + 4*h + r%4 ----
+        const uint32_t slot0 = b * 32u;
+        uint32_t mw = 0xffffffffu;
+        if (a.mask != nullptr) mw = uint32_t(a.mask[b >> 1] >> ((b & 1) * 32));
+        float vs[16];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            const float4 f = *reinterpret_cast<const float4 *>(a.scales + slot0 + 8 * q4 + 4 * h);
+            vs[q4 * 4 + 0] = f.x; vs[q4 * 4 + 1] = f.y; vs[q4 * 4 + 2] = f.z; vs[q4 * 4 + 3] = f.w;
+        }
+        if (DUMP) {
+            if (active) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int i = 8 * (r >> 2) + 4 * h + (r & 3);
+                    const uint32_t slot = slot0 + i;
+                    if (slot < a.n) {
+                        const float s = fmaf(float(acc[r]), qs, qb) * vs[r];
+                        const size_t o = size_t(qn) * a.n + slot;
+                        if (a.acc_out) a.acc_out[o] = acc[r];
+                        if (a.score_out) a.score_out[o] = ((mw >> i) & 1u) ? s : __int_as_float(0x7fc00000);
+                    }
+                }
+            }
+        } else {
+            if ((b & 3u) == 0u && lane < kQTile) atomicMax(&stau[lane], a.gtau[lane]);
+            const float tau = order_unkey(stau[qn]);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = 8 * (r >> 2) + 4 * h + (r & 3);
+                const uint32_t slot = slot0 + i;
+                const float s = fmaf(float(acc[r]), qs, qb) * vs[r];
+                if (active && s >= tau && (L.cnt < k || ranks_before(s, slot, L.worst_s, L.worst_i))) {
+                    if (slot < a.n && ((mw >> i) & 1u)) {
+                        if (list_offer(L, ls, li, kScanThreads, tid, k, s, slot)) {
+                            const int key = order_key(L.worst_s);
+                            if (atomicMax(&stau[qn], key) < key) atomicMax(&a.gtau[qn], key);
+                        }
+                    }
+                }
+            }
+        }
+        b = nb;
+    }
+
+    if (!DUMP) {
+        const size_t total_threads = size_t(gridDim.x) * kScanThreads;
+        const size_t gt = size_t(blockIdx.x) * kScanThreads + tid;
+        a.part_cnt[gt] = L.cnt;
+        for (int e = 0; e < L.cnt; ++e) {
+            a.part_scores[size_t(e) * total_threads + gt] = ls[e * kScanThreads + tid];
+            a.part_idx[size_t(e) * total_threads + gt] = li[e * kScanThreads + tid];
+        }
+    }
+}
+
+// ===========================================================================
+// Final merge of the per-lane lists of one query tile.
+// One workgroup per query: every thread folds a strided subset of the lists
+// into a private top-k, then the 256*k survivors are bitonic-sorted.
+// ===========================================================================
+
+__global__ __launch_bounds__(256) void k_merge(const float *__restrict__ part_scores,
+                                               const uint32_t *__restrict__ part_idx,
+                                               const int *__restrict__ part_cnt, int total_threads, int qmod,
+                                               int k, int k_eff, int sort_n, float *__restrict__ out_scores,
+                                               int64_t *__restrict__ out_idx) {
+    extern __shared__ __align__(16) uint8_t msm[];
+    float *ls = reinterpret_cast<float *>(msm);
+    uint32_t *li = reinterpret_cast<uint32_t *>(ls + k * 256);
+    uint64_t *keys = reinterpret_cast<uint64_t *>(li + k * 256);
+    __shared__ int total;
+    const int qn = blockIdx.x;
+    const int t = threadIdx.x;
+    if (t == 0) total = 0;
+    LaneList L{0, 0.0f, 0u, 0};
+    // lane (gt % 64) of every wave owns query (gt % 64) % qmod
+    const int per_wave = 64 / qmod;
+    const int n_lists = total_threads / 64 * per_wave;
+    for (int l = t; l < n_lists; l += 256) {
+        const int gt = (l / per_wave) * 64 + (l % per_wave) * qmod + qn;
+        const int cnt = part_cnt[gt];
+        for (int e = 0; e < cnt; ++e)
+            list_offer(L, ls, li, 256, t, k, part_scores[size_t(e) * total_threads + gt],
+                       part_idx[size_t(e) * total_threads + gt]);
+    }
+    __syncthreads();
+    const int base = atomicAdd(&total, L.cnt);
+    for (int e = 0; e < L.cnt; ++e) keys[base + e] = sort_key(ls[e * 256 + t], li[e * 256 + t]);
+    __syncthreads();
+    for (int i = total + t; i < sort_n; i += 256) keys[i] = 0;  // below every real key
+    __syncthreads();
+    for (int size = 2; size <= sort_n; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            for (int i = t; i < sort_n / 2; i += 256) {
+                const int lo = 2 * i - (i & (stride - 1));
+                const int hi = lo + stride;
+                const bool desc = (lo & size) == 0;
+                const uint64_t x = keys[lo], y = keys[hi];
+                if ((x < y) == desc) { keys[lo] = y; keys[hi] = x; }
+            }
+            __syncthreads();
+        }
+    }
+    for (int j = t; j < k_eff; j += 256) {
+        float s; uint32_t idx;
+        sort_unkey(keys[j], s, idx);
+        out_scores[size_t(qn) * k_eff + j] = s;
+        out_idx[size_t(qn) * k_eff + j] = int64_t(idx);
+    }
+}
+
+// ===========================================================================
+// Launchers
+// ===========================================================================
+
+hipError_t launch_seq_to_native(const uint8_t *d_seq, uint8_t *d_native, const Geometry &g, size_t first_block,
+                                size_t n_blocks, hipStream_t s) {
+    if (n_blocks == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_seq_to_native, dim3(unsigned(n_blocks * g.nch)), dim3(256), 0, s, d_seq, d_native, g.G,
+                       g.nch, first_block);
+    return hipGetLastError();
+}
+
+hipError_t launch_native_to_seq(const uint8_t *d_native, uint8_t *d_seq, const Geometry &g, size_t first_block,
+                                size_t n_blocks, hipStream_t s) {
+    if (n_blocks == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_native_to_seq, dim3(unsigned(n_blocks * g.nch)), dim3(256), 0, s, d_native, d_seq, g.G,
+                       g.nch, first_block);
+    return hipGetLastError();
+}
+
+hipError_t launch_append_rows(const uint8_t *d_rows, uint8_t *d_native, const Geometry &g, size_t old_n,
+                              size_t n_new, hipStream_t s) {
+    const size_t total = n_new * size_t(g.G);
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_append_rows, dim3(unsigned((total + 255) / 256)), dim3(256), 0, s, d_rows, d_native, g.G,
+                       g.nch, old_n, n_new);
+    return hipGetLastError();
+}
+
+hipError_t launch_move_lane(uint8_t *d_native, float *d_scales, const Geometry &g, size_t src, size_t dst,
+                            hipStream_t s) {
+    hipLaunchKernelGGL(k_move_lane, dim3(unsigned((g.G + 255) / 256)), dim3(256), 0, s, d_native, d_scales, g.G,
+                       g.nch, src, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_fill_i32(int *p, int v, size_t n, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_fill_i32, dim3(unsigned((n + 255) / 256)), dim3(256), 0, s, p, v, n);
+    return hipGetLastError();
+}
+
+template <typename K>
+static hipError_t allow_lds(K kernel, size_t bytes) {
+    if (bytes <= 48 * 1024) return hipSuccess;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               int(bytes));
+}
+
+hipError_t launch_rotate(const float *d_q, float *d_out, const float *d_signs, const uint32_t *d_perms, int dim,
+                         int block, float inv_sqrt_block, size_t nq, hipStream_t s) {
+    if (nq == 0) return hipSuccess;
+    const size_t lds = size_t(2) * dim * sizeof(float);
+    hipError_t e = allow_lds(k_rotate, lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(k_rotate, dim3(unsigned(nq)), dim3(256), lds, s, d_q, d_out, d_signs, d_perms, dim, block,
+                       inv_sqrt_block);
+    return hipGetLastError();
+}
+
+hipError_t launch_calibrate(const float *d_qrot, float *d_qcal, float *d_bias_corr, const float *d_shift,
+                            const float *d_scale, int dim, size_t nq, hipStream_t s) {
+    if (nq == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_calibrate, dim3(unsigned(nq)), dim3(256), 0, s, d_qrot, d_qcal, d_bias_corr, d_shift,
+                       d_scale, dim);
+    return hipGetLastError();
+}
+
+hipError_t launch_build_p(const float *d_qcal, const float *d_bias_corr, uint8_t *d_wfrag, float *d_qscale,
+                          float *d_qbias, int dim, int G, int nch, float cs, size_t nq, size_t nq_padded,
+                          hipStream_t s) {
+    if (nq_padded == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_build_p, dim3(unsigned(nq_padded)), dim3(256), 0, s, d_qcal, d_bias_corr, d_wfrag, d_qscale,
+                       d_qbias, dim, G, nch, cs, nq);
+    return hipGetLastError();
+}
+
+hipError_t launch_build_lut(const float *d_qcal, const float *d_bias_corr, const float *d_centroids, uint8_t *d_lut,
+                            float *d_qscale, float *d_qbias, int dim, int bits, int G, int nch, size_t nq,
+                            size_t nq_padded, hipStream_t s) {
+    if (nq_padded == 0) return hipSuccess;
+    const size_t lds = size_t(2) * G * sizeof(float);
+    hipError_t e = hipSuccess;
+#define TV_LAUNCH_LUT(B)                                                                                         \
+    e = allow_lds(k_build_lut<B>, lds);                                                                          \
+    if (e != hipSuccess) return e;                                                                               \
+    hipLaunchKernelGGL(k_build_lut<B>, dim3(unsigned(nq_padded)), dim3(256), lds, s, d_qcal, d_bias_corr,        \
+                       d_centroids, d_lut, d_qscale, d_qbias, dim, G, nch, nq)
+    if (bits == 2) { TV_LAUNCH_LUT(2); }
+    else if (bits == 3) { TV_LAUNCH_LUT(3); }
+    else { TV_LAUNCH_LUT(4); }
+#undef TV_LAUNCH_LUT
+    return hipGetLastError();
+}
+
+static constexpr size_t kLdsBudget = 160 * 1024;
+
+size_t scan_lds_bytes(int mode_p, int nch, int k, int lut_queries) {
+    const size_t lists = size_t(k) * kScanThreads * 8 + kQTile * sizeof(int);
+    if (mode_p) {
+        const size_t w = size_t(nch) * 2048;
+        return (w + lists <= kLdsBudget ? w : 0) + lists;
+    }
+    return size_t(nch) * 1024 * lut_queries + lists;
+}
+
+int scan_grid_blocks(int device, int mode_p, int nch, int k, int nq_tile) {
+    hipDeviceProp_t prop;
+    int cus = 256;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0)
+        cus = prop.multiProcessorCount;
+    const size_t lds = scan_lds_bytes(mode_p, nch, k, nq_tile);
+    int per_cu = int(kLdsBudget / (lds ? lds : 1));
+    if (per_cu < 1) per_cu = 1;
+    if (per_cu > 4) per_cu = 4;
+    return cus * per_cu;
+}
+
+hipError_t launch_scan_p4(const ScanArgs &a, int grid, bool dump, hipStream_t s) {
+    const size_t w = size_t(a.nch) * 2048;
+    const size_t lists = dump ? 64 : size_t(a.k) * kScanThreads * 8 + kQTile * sizeof(int);
+    const bool w_lds = w + lists <= kLdsBudget;
+    const size_t lds = (w_lds ? w : 0) + lists;
+    hipError_t e = hipSuccess;
+#define TV_LAUNCH_P4(U, D, W)                                                                   \
+    do {                                                                                        \
+        e = allow_lds(k_scan_p4<U, D, W>, lds);                                                 \
+        if (e != hipSuccess) return e;                                                          \
+        hipLaunchKernelGGL((k_scan_p4<U, D, W>), dim3(grid), dim3(kScanThreads), lds, s, a);    \
+    } while (0)
+#define TV_PICK_P4(U)                                                                           \
+    do {                                                                                        \
+        if (dump) { if (w_lds) TV_LAUNCH_P4(U, true, true); else TV_LAUNCH_P4(U, true, false); } \
+        else { if (w_lds) TV_LAUNCH_P4(U, false, true); else TV_LAUNCH_P4(U, false, false); }   \
+    } while (0)
+    if (a.nch % 4 == 0) TV_PICK_P4(4);
+    else if (a.nch % 2 == 0) TV_PICK_P4(2);
+    else TV_PICK_P4(1);
+#undef TV_PICK_P4
+#undef TV_LAUNCH_P4
+    return hipGetLastError();
+}
+
+hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, const int *part_cnt, int total_threads,
+                        int qmod, int k, int k_eff, int nq_tile, float *out_scores, int64_t *out_idx,
+                        hipStream_t s) {
+    if (nq_tile == 0 || k_eff == 0) return hipSuccess;
+    int sort_n = 2;
+    while (sort_n < 256 * k) sort_n <<= 1;
+    const size_t lds = size_t(k) * 256 * 8 + size_t(sort_n) * 8;
+    hipError_t e = allow_lds(k_merge, lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(k_merge, dim3(nq_tile), dim3(256), lds, s, part_scores, part_idx, part_cnt, total_threads,
+                       qmod, k, k_eff, sort_n, out_scores, out_idx);
+    return hipGetLastError();
+}
+
+}  // namespace tv
