@@ -81,6 +81,8 @@ int tv_index_get_tables(const tv_index *ix, float *signs, uint32_t *perms, float
  * lane l) at (b*G+g)*32+l, ceil(n/32)*G*32 bytes) and their per-vector scales
  * (lib.rs:312).  Replaces BlockedCache (lib.rs:253-256). */
 int tv_index_upload_seq(tv_index *ix, const uint8_t *seq_codes, size_t n_vectors, const float *scales);
+/* Same, from device memory (both pointers are device pointers). */
+int tv_index_upload_seq_dev(tv_index *ix, const uint8_t *d_seq_codes, size_t n_vectors, const float *d_scales);
 /* Append n_new rows; rows[i*G + g] is row i's code byte of group g (the
  * per-vector form extract_codes_flat yields, pack.rs:306).  Replaces
  * append_lanes (pack.rs:211-233). */
@@ -120,6 +122,13 @@ int tv_search(tv_index *ix, const float *queries, size_t nq, size_t k,
 int tv_search_dev(tv_index *ix, const float *d_queries, size_t nq, size_t k,
                   const uint64_t *d_mask_words, size_t n_allowed,
                   float *d_out_scores, int64_t *d_out_indices, size_t *out_k_eff);
+
+/* ---- host-only derivations (no GPU touched) ------------------------------- */
+
+/* The tables tv_index_create derives: Rotation::new (rotation.rs:141-187;
+ * signs/perms 2*dim each, round 0 first) and codebook::codebook (codebook.rs:50). */
+int tv_host_rotation_tables(int dim, float *signs, uint32_t *perms, int *block, float *inv_sqrt_block);
+int tv_host_codebook(int bits, int dim, float *boundaries, float *centroids);
 
 /* ---- test / measurement hooks -------------------------------------------- */
 

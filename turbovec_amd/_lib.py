@@ -27,9 +27,9 @@ SCORE_AUTO, SCORE_L_CLASSIC, SCORE_L_U32, SCORE_P = 0, 2, 3, 4
 EXPORTS = [
     "tv_status_string", "tv_last_error", "tv_index_create", "tv_index_destroy", "tv_index_set_tables",
     "tv_index_set_calibration", "tv_index_set_score_mode", "tv_index_get_tables", "tv_index_upload_seq",
-    "tv_index_append_rows", "tv_index_swap_remove", "tv_index_download_seq", "tv_index_len", "tv_index_dim",
+    "tv_index_upload_seq_dev", "tv_index_append_rows", "tv_index_swap_remove", "tv_index_download_seq", "tv_index_len", "tv_index_dim",
     "tv_index_bits", "tv_validate_queries", "tv_pack_mask", "tv_search", "tv_search_dev", "tv_debug_scan",
-    "tv_debug_prepare", "tv_last_scan_ms", "tv_index_device_ptrs",
+    "tv_debug_prepare", "tv_last_scan_ms", "tv_index_device_ptrs", "tv_host_rotation_tables", "tv_host_codebook",
 ]
 
 _lib = None
@@ -62,6 +62,7 @@ def lib():
     L.tv_index_set_score_mode.argtypes = [vp, i32]
     L.tv_index_get_tables.argtypes = [vp, vp, vp, vp, vp]
     L.tv_index_upload_seq.argtypes = [vp, vp, sz, vp]
+    L.tv_index_upload_seq_dev.argtypes = [vp, vp, sz, vp]
     L.tv_index_append_rows.argtypes = [vp, vp, vp, sz]
     L.tv_index_swap_remove.argtypes = [vp, sz]
     L.tv_index_download_seq.argtypes = [vp, vp, vp]
@@ -77,6 +78,8 @@ def lib():
     L.tv_debug_prepare.argtypes = [vp, vp, sz, vp, vp, vp]
     L.tv_last_scan_ms.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(i32)]
     L.tv_index_device_ptrs.argtypes = [vp, C.POINTER(vp), C.POINTER(vp), C.POINTER(sz)]
+    L.tv_host_rotation_tables.argtypes = [i32, vp, vp, C.POINTER(i32), C.POINTER(C.c_float)]
+    L.tv_host_codebook.argtypes = [i32, i32, vp, vp]
     _lib = L
     return L
 
@@ -104,9 +107,9 @@ class NativeIndex:
         self.n_byte_groups = dim // (8 // bits)
 
     def close(self):
-        if getattr(self, "h", None):
-            lib().tv_index_destroy(self.h)
-            self.h = None
+        h, self.h = getattr(self, "h", None), None
+        if h and _lib is not None:
+            _lib.tv_index_destroy(h)
 
     __del__ = close
 
@@ -145,6 +148,9 @@ class NativeIndex:
         assert seq.size == ((n + 31) // 32) * self.n_byte_groups * 32, "sequential-blocked size mismatch"
         assert sc.size == n
         check(lib().tv_index_upload_seq(self.h, ptr(seq), n, ptr(sc)))
+
+    def upload_seq_dev(self, d_seq_ptr, n, d_scales_ptr):
+        check(lib().tv_index_upload_seq_dev(self.h, d_seq_ptr, n, d_scales_ptr))
 
     def append_rows(self, rows, scales):
         r = np.ascontiguousarray(rows, np.uint8).reshape(-1, self.n_byte_groups)
@@ -226,3 +232,21 @@ def pack_mask(mask_bytes):
     allowed = C.c_size_t(0)
     check(lib().tv_pack_mask(ptr(m), m.size, ptr(words), C.byref(allowed)))
     return words, allowed.value
+
+
+def host_rotation_tables(dim):
+    """The rotation tables the library derives for `dim` (no GPU needed)."""
+    signs = np.zeros((2, dim), np.float32)
+    perms = np.zeros((2, dim), np.uint32)
+    block = C.c_int(0)
+    inv = C.c_float(0)
+    check(lib().tv_host_rotation_tables(dim, ptr(signs), ptr(perms), C.byref(block), C.byref(inv)))
+    return signs, perms, block.value, np.float32(inv.value)
+
+
+def host_codebook(bits, dim):
+    """(boundaries, centroids) the library derives (no GPU needed)."""
+    b = np.zeros((1 << bits) - 1, np.float32)
+    c = np.zeros(1 << bits, np.float32)
+    check(lib().tv_host_codebook(bits, dim, ptr(b), ptr(c)))
+    return b, c

@@ -439,6 +439,30 @@ int tv_index_upload_seq(tv_index *ix, const uint8_t *seq_codes, size_t n_vectors
     return TV_OK;
 }
 
+int tv_index_upload_seq_dev(tv_index *ix, const uint8_t *d_seq_codes, size_t n_vectors, const float *d_scales) {
+    if (!ix || (n_vectors && (!d_seq_codes || !d_scales))) return TV_ERR_BAD_ARGUMENT;
+    if (n_vectors >= (size_t(1) << 31)) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    ix->n = 0;
+    int rc = ensure_capacity(ix, n_vectors);
+    if (rc != TV_OK) return rc;
+    const size_t n_blocks = (n_vectors + tv::kVecBlock - 1) / tv::kVecBlock;
+    const size_t seq_block = size_t(ix->geo.G) * tv::kVecBlock;
+    const size_t slice_blocks = std::max<size_t>(1, (size_t(1) << 30) / seq_block);  // keeps each grid small
+    for (size_t b0 = 0; b0 < n_blocks; b0 += slice_blocks) {
+        const size_t nb = std::min(slice_blocks, n_blocks - b0);
+        TV_HIP(tv::launch_seq_to_native(d_seq_codes + b0 * seq_block, ix->d_codes, ix->geo, b0, nb, ix->stream));
+    }
+    if (n_vectors) {
+        TV_HIP(hipMemsetAsync(ix->d_scales, 0, n_blocks * tv::kVecBlock * sizeof(float), ix->stream));
+        TV_HIP(hipMemcpyAsync(ix->d_scales, d_scales, n_vectors * sizeof(float), hipMemcpyDeviceToDevice, ix->stream));
+    }
+    TV_HIP(hipStreamSynchronize(ix->stream));
+    ix->n = n_vectors;
+    return TV_OK;
+}
+
 int tv_index_append_rows(tv_index *ix, const uint8_t *rows, const float *scales, size_t n_new) {
     if (!ix || (n_new && (!rows || !scales))) return TV_ERR_BAD_ARGUMENT;
     if (n_new == 0) return TV_OK;
@@ -660,6 +684,24 @@ int tv_debug_prepare(tv_index *ix, const float *queries, size_t nq, float *q_rot
     if (scale_out) TV_HIP(hipMemcpyAsync(scale_out, pq.d_qscale, nq * 4, hipMemcpyDeviceToHost, ix->stream));
     if (bias_out) TV_HIP(hipMemcpyAsync(bias_out, pq.d_qbias, nq * 4, hipMemcpyDeviceToHost, ix->stream));
     TV_HIP(hipStreamSynchronize(ix->stream));
+    return TV_OK;
+}
+
+int tv_host_rotation_tables(int dim, float *signs, uint32_t *perms, int *block, float *inv_sqrt_block) {
+    if (dim <= 0 || dim % 8 != 0 || dim > 16384) return TV_ERR_BAD_ARGUMENT;
+    const tv::RotationTables t = tv::make_rotation_tables(dim);
+    if (signs) std::memcpy(signs, t.signs.data(), t.signs.size() * sizeof(float));
+    if (perms) std::memcpy(perms, t.perms.data(), t.perms.size() * sizeof(uint32_t));
+    if (block) *block = t.block;
+    if (inv_sqrt_block) *inv_sqrt_block = t.inv_sqrt_block;
+    return TV_OK;
+}
+
+int tv_host_codebook(int bits, int dim, float *boundaries, float *centroids) {
+    if (bits < 2 || bits > 4 || dim < 8 || dim > 16384) return TV_ERR_BAD_ARGUMENT;
+    const tv::Codebook cb = tv::make_codebook(bits, dim);
+    if (boundaries) std::memcpy(boundaries, cb.boundaries.data(), cb.boundaries.size() * sizeof(float));
+    if (centroids) std::memcpy(centroids, cb.centroids.data(), cb.centroids.size() * sizeof(float));
     return TV_OK;
 }
 
