@@ -66,6 +66,7 @@ def _load():
     lib.tvo_calibrate_query.argtypes = [f32p, f32p, f32p, i32, f32p, f32p]
     lib.tvo_search.argtypes = [i32, f32p, sz, vp, vp, f32p, f32p, f32p, f32p, i32, i32, sz, sz, vp,
                                f32p, vp, vp, vp, f32p, i32]
+    lib.tvo_search_fast.argtypes = [f32p, sz, vp, vp, f32p, f32p, i32, i32, sz, sz, vp, f32p, vp, vp, i32]
     lib.tvo_validate_queries.argtypes = [f32p, sz, i32, vp]
     lib.tvo_pack_mask.restype = sz
     lib.tvo_pack_mask.argtypes = [vp, sz, vp]
@@ -263,6 +264,29 @@ def search(rot, seq, scales, queries, k, bits, dim, n, mask_words=None, mode=MOD
     assert k_eff.value == kk, (k_eff.value, kk)
     if dump:
         return out_s, out_i, acc, sc
+    return out_s, out_i
+
+
+def search_fast(rot, seq, scales, queries, k, bits, dim, n, mask_words=None, n_threads=8):
+    """Throughput-oriented twin of search() (modes P / L_U32, uncalibrated, k <= 1024)."""
+    q = _f32(queries).reshape(-1, dim)
+    nq = q.shape[0]
+    _, cen = codebook(bits, dim)
+    seq = np.ascontiguousarray(seq, np.uint8)
+    scales = _f32(scales)
+    n_allowed = n
+    if mask_words is not None:
+        mask_words = np.ascontiguousarray(mask_words, np.uint64)
+        n_allowed = int(np.unpackbits(mask_words.view(np.uint8)).sum())
+    kk = min(k, n, n_allowed)
+    assert kk <= 1024
+    out_s = np.zeros((nq, kk), np.float32)
+    out_i = np.zeros((nq, kk), np.int64)
+    k_eff = C.c_size_t(0)
+    rc = lib().tvo_search_fast(_p(q), nq, rot.h, _p(seq), _p(cen), _p(scales), bits, dim, n, k,
+                               _p(mask_words), _p(out_s), _p(out_i), C.addressof(k_eff), n_threads)
+    if rc != 0:
+        raise RuntimeError(f"tvo_search_fast failed rc={rc}")
     return out_s, out_i
 
 

@@ -818,6 +818,172 @@ int tvo_search(int mode, const float *queries, size_t nq, const tvo_rotation *ro
 }
 
 /* ======================================================================= */
+/* Throughput-oriented variant for the CPU baseline: same results as        */
+/* tvo_search in modes P and L_U32 (tests compare them), organised like the */
+/* reference's batch path (search.rs:4005-4050): block ranges are split     */
+/* across threads, each block's codes are decoded once and reused by every  */
+/* query, per-range heaps are merged by (score desc, slot asc).             */
+/* ======================================================================= */
+
+typedef struct {
+    float *hs; uint64_t *hi; size_t sz, mi; float mn;
+} heap_t;
+
+static inline void heap_push(heap_t *h, size_t k, float score, uint64_t vi) {
+    if (h->sz < k) {
+        h->hs[h->sz] = score; h->hi[h->sz] = vi; h->sz++;
+        if (h->sz == k) rescan_min(h->hs, h->hi, k, &h->mn, &h->mi);
+    } else if (score > h->mn) {
+        h->hs[h->mi] = score; h->hi[h->mi] = vi;
+        rescan_min(h->hs, h->hi, k, &h->mn, &h->mi);
+    }
+}
+
+__attribute__((target_clones("arch=skylake-avx512", "avx2", "default")))
+int32_t tvo_dot_i8(const int8_t *a, const int8_t *b, int n) {
+    int32_t s = 0;
+    for (int i = 0; i < n; i++) s += (int32_t)a[i] * (int32_t)b[i];
+    return s;
+}
+
+int tvo_search_fast(const float *queries, size_t nq, const tvo_rotation *rot,
+                    const uint8_t *seq, const float *centroids, const float *vec_scales,
+                    int bits, int dim, size_t n, size_t k, const uint64_t *mask,
+                    float *out_scores, int64_t *out_indices, size_t *out_k_eff, int n_threads) {
+    size_t G = tvo_n_byte_groups(bits, dim);
+    size_t n_blocks = (n + TVO_BLOCK - 1) / TVO_BLOCK;
+    size_t n_allowed = n;
+    if (mask) {
+        n_allowed = 0;
+        for (size_t w = 0; w < (n + 63) / 64; w++) n_allowed += (size_t)__builtin_popcountll(mask[w]);
+    }
+    if (k > n_allowed) k = n_allowed;
+    if (k > n) k = n;
+    *out_k_eff = k;
+    if (k == 0 || nq == 0) return TVO_OK;
+    if (n_threads < 1) n_threads = 1;
+    const int mode_p = bits == 4;
+    /* per-query tables */
+    int8_t *W = NULL; uint8_t *LUT = NULL; int8_t levels[16];
+    float *qscale = (float *)malloc(sizeof(float) * nq), *qbias = (float *)malloc(sizeof(float) * nq);
+    if (mode_p) W = (int8_t *)malloc(nq * (size_t)dim); else LUT = (uint8_t *)malloc(nq * G * 32);
+#pragma omp parallel for schedule(static) num_threads(n_threads)
+    for (long long qi = 0; qi < (long long)nq; qi++) {
+        float *q_rot = (float *)malloc(sizeof(float) * (size_t)dim);
+        memcpy(q_rot, queries + (size_t)qi * dim, sizeof(float) * (size_t)dim);
+        tvo_rotation_apply(rot, q_rot);
+        if (mode_p) {
+            int8_t *w = (int8_t *)malloc((size_t)dim); int32_t zero; int8_t lv[16];
+            tvo_build_permute_dot(q_rot, centroids, dim, lv, w, &zero, &qscale[qi]);
+            if (qi == 0) memcpy(levels, lv, 16);
+            qbias[qi] = 0.0f;
+            int8_t *dst = W + (size_t)qi * dim;      /* per-dimension order */
+            for (size_t g = 0; g < G; g++) {
+                dst[2 * g + 1] = w[(g / 4) * 8 + g % 4];
+                dst[2 * g] = w[(g / 4) * 8 + 4 + g % 4];
+            }
+            free(w);
+        } else {
+            tvo_build_lut(q_rot, centroids, bits, dim, LUT + (size_t)qi * G * 32, &qscale[qi], &qbias[qi]);
+        }
+        free(q_rot);
+    }
+    if (mode_p && nq > 0) { /* levels are query independent; make sure thread 0's copy is visible */
+        float cmax = 0.0f;
+        for (int i = 0; i < 16; i++) { float v = fabsf(centroids[i]); if (v > cmax) cmax = v; }
+        float cs = cmax > 0.0f ? cmax / 127.0f : 1.0f;
+        for (int i = 0; i < 16; i++) levels[i] = (int8_t)clampf(roundf(centroids[i] / cs), -127.0f, 127.0f);
+    }
+    /* block ranges: even block counts so ranges start on mask-word boundaries (search.rs:3038) */
+    size_t n_ranges = (size_t)n_threads * 4;
+    size_t stride = (n_blocks + n_ranges - 1) / n_ranges;
+    if (stride < 2) stride = 2;
+    stride += stride & 1;
+    n_ranges = (n_blocks + stride - 1) / stride;
+    float *all_s = (float *)malloc(sizeof(float) * n_ranges * nq * k);
+    uint64_t *all_i = (uint64_t *)malloc(sizeof(uint64_t) * n_ranges * nq * k);
+    size_t *all_sz = (size_t *)calloc(n_ranges * nq, sizeof(size_t));
+#pragma omp parallel for schedule(dynamic, 1) num_threads(n_threads)
+    for (long long r = 0; r < (long long)n_ranges; r++) {
+        size_t b0 = (size_t)r * stride, b1 = b0 + stride < n_blocks ? b0 + stride : n_blocks;
+        heap_t *heaps = (heap_t *)malloc(sizeof(heap_t) * nq);
+        for (size_t qi = 0; qi < nq; qi++) {
+            heaps[qi].hs = all_s + ((size_t)r * nq + qi) * k;
+            heaps[qi].hi = all_i + ((size_t)r * nq + qi) * k;
+            heaps[qi].sz = 0; heaps[qi].mi = 0; heaps[qi].mn = -INFINITY;
+        }
+        int8_t *dec = mode_p ? (int8_t *)malloc((size_t)TVO_BLOCK * (size_t)dim) : NULL;
+        for (size_t b = b0; b < b1; b++) {
+            size_t base_vec = b * TVO_BLOCK;
+            uint32_t mw = 0xFFFFFFFFu;
+            if (mask) { mw = (uint32_t)(mask[base_vec >> 6] >> (base_vec & 63)); if (!mw) continue; }
+            size_t lanes = n - base_vec < TVO_BLOCK ? n - base_vec : TVO_BLOCK;
+            const uint8_t *blk = seq + b * G * TVO_BLOCK;
+            if (mode_p) {
+                for (size_t g = 0; g < G; g++)
+                    for (size_t l = 0; l < lanes; l++) {
+                        unsigned byte = blk[g * TVO_BLOCK + l];
+                        dec[l * (size_t)dim + 2 * g] = levels[byte >> 4];
+                        dec[l * (size_t)dim + 2 * g + 1] = levels[byte & 15];
+                    }
+                for (size_t qi = 0; qi < nq; qi++) {
+                    const int8_t *w = W + qi * (size_t)dim;
+                    for (size_t l = 0; l < lanes; l++) {
+                        if (!((mw >> l) & 1)) continue;
+                        int32_t acc = tvo_dot_i8(w, dec + l * (size_t)dim, dim);
+                        float score = fmaf((float)acc, qscale[qi], qbias[qi]) * vec_scales[base_vec + l];
+                        heap_push(&heaps[qi], k, score, base_vec + l);
+                    }
+                }
+            } else {
+                for (size_t qi = 0; qi < nq; qi++) {
+                    const uint8_t *lut = LUT + qi * G * 32;
+                    uint32_t acc[TVO_BLOCK] = {0};
+                    for (size_t g = 0; g < G; g++) {
+                        const uint8_t *row = lut + g * 32;
+                        const uint8_t *cb = blk + g * TVO_BLOCK;
+                        for (size_t l = 0; l < TVO_BLOCK; l++) acc[l] += (uint32_t)row[cb[l] >> 4] + (uint32_t)row[16 + (cb[l] & 15)];
+                    }
+                    for (size_t l = 0; l < lanes; l++) {
+                        if (!((mw >> l) & 1)) continue;
+                        float score = (((float)(int32_t)acc[l] * qscale[qi]) + qbias[qi]) * vec_scales[base_vec + l];
+                        heap_push(&heaps[qi], k, score, base_vec + l);
+                    }
+                }
+            }
+        }
+        for (size_t qi = 0; qi < nq; qi++) all_sz[(size_t)r * nq + qi] = heaps[qi].sz;
+        free(dec); free(heaps);
+    }
+    int err = 0;
+#pragma omp parallel for schedule(static) num_threads(n_threads)
+    for (long long qi = 0; qi < (long long)nq; qi++) {
+        pair_t *pairs = (pair_t *)malloc(sizeof(pair_t) * n_ranges * k);
+        size_t np = 0;
+        for (size_t r = 0; r < n_ranges; r++) {
+            size_t sz = all_sz[r * nq + (size_t)qi];
+            for (size_t j = 0; j < sz; j++) {
+                pairs[np].s = all_s[(r * nq + (size_t)qi) * k + j];
+                pairs[np].i = all_i[(r * nq + (size_t)qi) * k + j];
+                np++;
+            }
+        }
+        qsort(pairs, np, sizeof(pair_t), cmp_pair);          /* search.rs:4279-4298 */
+        if (np < k) {
+#pragma omp atomic write
+            err = 1;
+        }
+        for (size_t j = 0; j < k && j < np; j++) {
+            out_scores[(size_t)qi * k + j] = pairs[j].s;
+            out_indices[(size_t)qi * k + j] = (int64_t)pairs[j].i;
+        }
+        free(pairs);
+    }
+    free(all_s); free(all_i); free(all_sz); free(qscale); free(qbias); free(W); free(LUT);
+    return err ? TVO_ERR_BAD_ARGUMENT : TVO_OK;
+}
+
+/* ======================================================================= */
 /* Fixture helpers                                                          */
 /* ======================================================================= */
 

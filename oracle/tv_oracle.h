@@ -146,6 +146,15 @@ int tvo_search(int mode, const float *queries, size_t nq, const tvo_rotation *ro
                float *out_scores, int64_t *out_indices, size_t *out_k_eff,
                int32_t *acc_dump, float *score_dump, int n_threads);
 
+/* Same answer as tvo_search in the modes a VNNI host runs (P at 4-bit, L_U32
+ * otherwise), uncalibrated indexes, k <= 1024; organised for throughput (block
+ * ranges over threads, codes decoded once per block, per-range heaps merged as
+ * search.rs:4279-4298 does).  This is what the CPU-baseline timing runs. */
+int tvo_search_fast(const float *queries, size_t nq, const tvo_rotation *rot,
+                    const uint8_t *seq_codes, const float *centroids, const float *vec_scales,
+                    int bits, int dim, size_t n, size_t k, const uint64_t *mask_words,
+                    float *out_scores, int64_t *out_indices, size_t *out_k_eff, int n_threads);
+
 /* Caller-side checks that precede the seam (turbovec/src/lib.rs:1363-1380,
  * encode.rs:76-83): returns TVO_OK or the error; *bad_index = flat offset. */
 int tvo_validate_queries(const float *queries, size_t len, int dim, size_t *bad_index);

@@ -414,3 +414,22 @@ def test_query_validation(oracle):
     q2 = q.copy()
     q2[3] = np.float32(9.99e15)
     assert O.validate_queries(q2, 8)[0] == O.OK
+
+
+# The throughput-oriented twin the CPU baseline times must give the same answer.
+@pytest.mark.parametrize("dim,bits,n", [(1536, 4, 3000), (1536, 2, 3000), (128, 4, 5003), (64, 3, 700)])
+def test_search_fast_equals_search(oracle, dim, bits, n):
+    O = oracle
+    rng = np.random.default_rng(21)
+    v = rng.standard_normal((n, dim)).astype(np.float32)
+    q = rng.standard_normal((37, dim)).astype(np.float32)
+    rot = O.Rotation(dim)
+    packed, scales = O.encode(rot, v, bits)
+    seq = O.repack_seq(packed, n, bits, dim)
+    s, i = O.search(rot, seq, scales, q, 10, bits, dim, n)
+    s2, i2 = O.search_fast(rot, seq, scales, q, 10, bits, dim, n, n_threads=4)
+    assert np.array_equal(i, i2) and _eq_bits(s, s2)
+    words, _ = O.pack_mask(rng.random(n) < 0.03)
+    s, i = O.search(rot, seq, scales, q, 10, bits, dim, n, mask_words=words)
+    s2, i2 = O.search_fast(rot, seq, scales, q, 10, bits, dim, n, mask_words=words, n_threads=3)
+    assert np.array_equal(i, i2) and _eq_bits(s, s2)
