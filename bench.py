@@ -36,6 +36,8 @@ def parse():
     ap.add_argument("--batch", type=int, default=1024)
     ap.add_argument("--cpu-sample", type=int, default=2_000_000, help="vectors in the CPU-baseline sample (0 = skip)")
     ap.add_argument("--cpu-threads", type=int, default=16)
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="only run the plain copy kernel over a 4 GiB buffer (counter calibration) and exit")
     return ap.parse_args()
 
 
@@ -85,6 +87,15 @@ def main():
     from turbovec_amd import _lib as T
 
     dev = torch.device("cuda:0")
+    if args.copy_probe:
+        nbytes = 4 << 30
+        src = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+        dst = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        ix = T.NativeIndex(64, 4)
+        ms = ix.stream_probe(src.data_ptr(), dst.data_ptr(), nbytes, reps=3)
+        print(json.dumps({"copy_probe_bytes_read": nbytes, "copy_probe_bytes_written": nbytes, "ms": ms,
+                          "GBps_read_plus_write": 2 * nbytes / (ms * 1e-3) / 1e9}))
+        return
     n, dim, bits, k = args.n, args.dim, args.bits, args.k
     G = dim // (8 // bits)
     n_blocks = (n + 31) // 32
@@ -121,6 +132,9 @@ def main():
         return dt, scan_ms, launches
 
     alg_bytes = n_blocks * G * 32 + 4 * n          # codes + per-vector scales, one pass
+    d_codes, _, code_bytes = ix.device_ptrs()
+    read_ms = ix.stream_probe(d_codes, None, code_bytes, reps=5)   # pure read of the same buffer
+    read_probe = code_bytes / (read_ms * 1e-3) / 1e9
     dt, scan_ms, launches = run(args.batch, args.steps, args.warmup)
     value = args.batch * args.steps / dt
     launch_s = scan_ms * 1e-3 / max(launches, 1)
@@ -155,10 +169,12 @@ def main():
                    else "u8 LUT, u32 accumulate", "n": n, "dim": dim, "bits": bits, "k": k, "batch": args.batch},
         "batch1": {"queries_per_s": b1_steps / dt1, "ms_per_query": dt1 / b1_steps * 1e3,
                    "scan_kernel_ms": b1_launch_s * 1e3, "achieved_GBps": alg_bytes / b1_launch_s / 1e9,
-                   "frac_of_hbm_peak": alg_bytes / b1_launch_s / 1e9 / 8000.0},
+                   "frac_of_hbm_peak": alg_bytes / b1_launch_s / 1e9 / 8000.0,
+                   "frac_of_achievable": alg_bytes / b1_launch_s / 1e9 / read_probe},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s",
                      "frac": achieved / 8000.0, "traffic": traffic,
                      "kernel": "k_scan_p4" if bits == 4 else "k_scan_lut",
+                     "achievable_read_GBps": read_probe, "frac_of_achievable": achieved / read_probe,
                      "algorithmic_bytes_per_launch": alg_bytes, "launches_timed": launches,
                      "mean_launch_ms": launch_s * 1e3, "queries_per_launch": 32 if bits == 4 else None},
     }

@@ -143,6 +143,11 @@ int tv_debug_prepare(tv_index *ix, const float *queries, size_t nq,
  * tv_search* call on this index, measured with HIP events on its stream, and
  * how many launches that was. */
 int tv_last_scan_ms(const tv_index *ix, float *ms, int *launches);
+/* Bandwidth probe on the index's stream: reps launches of a pure read-sum over
+ * d_src (d_dst NULL) or of a plain copy d_src -> d_dst, bytes each; mean
+ * milliseconds per launch.  Calibrates the achievable HBM rate and gives the
+ * hardware counters a kernel of known traffic. */
+int tv_debug_stream_probe(tv_index *ix, const void *d_src, void *d_dst, size_t bytes, int reps, float *ms_per_rep);
 /* Device pointers of the resident index (native layout) for tools. */
 int tv_index_device_ptrs(const tv_index *ix, void **d_codes, void **d_scales, size_t *code_bytes);
 

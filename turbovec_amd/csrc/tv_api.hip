@@ -705,6 +705,26 @@ int tv_host_codebook(int bits, int dim, float *boundaries, float *centroids) {
     return TV_OK;
 }
 
+int tv_debug_stream_probe(tv_index *ix, const void *d_src, void *d_dst, size_t bytes, int reps, float *ms_per_rep) {
+    if (!ix || !d_src || reps <= 0) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    int rc = ensure_events();
+    if (rc != TV_OK) return rc;
+    rc = ensure_workspace(ix, 4096);
+    if (rc != TV_OK) return rc;
+    uint32_t *sink = static_cast<uint32_t *>(ix->ws);
+    TV_HIP(tv::launch_probe(d_src, d_dst, bytes, d_dst != nullptr, sink, ix->stream));  // warm
+    TV_HIP(hipEventRecord(g_events.start[0], ix->stream));
+    for (int r = 0; r < reps; ++r) TV_HIP(tv::launch_probe(d_src, d_dst, bytes, d_dst != nullptr, sink, ix->stream));
+    TV_HIP(hipEventRecord(g_events.stop[0], ix->stream));
+    TV_HIP(hipStreamSynchronize(ix->stream));
+    float ms = 0.0f;
+    TV_HIP(hipEventElapsedTime(&ms, g_events.start[0], g_events.stop[0]));
+    if (ms_per_rep) *ms_per_rep = ms / float(reps);
+    return TV_OK;
+}
+
 int tv_last_scan_ms(const tv_index *ix, float *ms, int *launches) {
     if (!ix) return TV_ERR_BAD_ARGUMENT;
     if (ms) *ms = ix->last_scan_ms;

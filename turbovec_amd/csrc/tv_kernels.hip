@@ -522,6 +522,38 @@ __global__ __launch_bounds__(256) void k_merge(const float *__restrict__ part_sc
 }
 
 // ===========================================================================
+// Bandwidth probes: a pure read (sum) and a plain copy over a caller buffer.
+// They calibrate what the scan can hope for on this device and give the
+// hardware counters a kernel of known traffic to be scaled against.
+// ===========================================================================
+
+__global__ __launch_bounds__(256) void k_probe_read(const uint4 *__restrict__ src, size_t n16, uint32_t *sink) {
+    uint32_t acc = 0;
+    size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+    const size_t stride = size_t(gridDim.x) * 256;
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+        const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+        acc += a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    }
+    for (; i < n16; i += stride) { const uint4 a = src[i]; acc += a.x ^ a.y ^ a.z ^ a.w; }
+    if (acc == 0x12345678u) *sink = acc;  // keeps the loads alive; practically never taken
+}
+
+__global__ __launch_bounds__(256) void k_probe_copy(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16) {
+    size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+    const size_t stride = size_t(gridDim.x) * 256;
+    for (; i < n16; i += stride) dst[i] = src[i];
+}
+
+hipError_t launch_probe(const void *src, void *dst, size_t bytes, int copy, uint32_t *sink, hipStream_t s) {
+    const size_t n16 = bytes / 16;
+    if (copy) hipLaunchKernelGGL(k_probe_copy, dim3(256 * 8), dim3(256), 0, s, static_cast<const uint4 *>(src),
+                                 static_cast<uint4 *>(dst), n16);
+    else hipLaunchKernelGGL(k_probe_read, dim3(256 * 8), dim3(256), 0, s, static_cast<const uint4 *>(src), n16, sink);
+    return hipGetLastError();
+}
+
+// ===========================================================================
 // Launchers
 // ===========================================================================
 
