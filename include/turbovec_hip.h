@@ -143,6 +143,13 @@ int tv_debug_prepare(tv_index *ix, const float *queries, size_t nq,
  * tv_search* call on this index, measured with HIP events on its stream, and
  * how many launches that was. */
 int tv_last_scan_ms(const tv_index *ix, float *ms, int *launches);
+/* Path selection for tests: non-zero makes every search take the full-range
+ * list / dense-select path instead of sample-then-filter (results must be
+ * identical either way). */
+int tv_debug_set_path(tv_index *ix, int force_full_lists);
+/* How many queries so far had to be redone through that path because their
+ * candidate buffer overflowed. */
+int tv_debug_overflow_redos(const tv_index *ix, size_t *count);
 /* Bandwidth probe on the index's stream: reps launches of a pure read-sum over
  * d_src (d_dst NULL) or of a plain copy d_src -> d_dst, bytes each; mean
  * milliseconds per launch.  Calibrates the achievable HBM rate and gives the

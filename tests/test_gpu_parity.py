@@ -442,3 +442,67 @@ def test_config2_scale_properties(T):
         order = order[m[order]][:10]
         assert im[qi].tolist() == order.tolist()
     ix.close()
+
+
+# ---- sample-then-filter path (n above the candidate capacity) ----
+@pytest.mark.parametrize("bits,mode", [(4, "P"), (2, "L_U32"), (4, "L_CLASSIC")])
+def test_sampled_path_matches_oracle_and_full_path(T, oracle, bits, mode):
+    O = oracle
+    dim, n, nq = 128, 40_003, 37
+    oidx = OracleIndex(O, dim, bits, unit_gaussian(n, dim, seed=31))
+    q = unit_gaussian(nq, dim, seed=32)
+    ix = to_native(T, oidx, tmode(T, mode))
+    rng = np.random.default_rng(5)
+    masks = [None, rng.random(n) < 0.5, rng.random(n) < 0.01, (np.arange(n) > 30_000) & (np.arange(n) < 32_000)]
+    for m in masks:
+        words = None if m is None else T.pack_mask(m)[0]
+        for k in (1, 10, 32, 33, 100, 1000, 1500):
+            s, i = ix.search(q, k, mask_words=words)
+            os_, oi = oidx.search(q, k, mask_words=words, mode=omode(O, mode))
+            assert np.array_equal(i, oi), (mode, k)
+            assert bits_equal(s, os_), (mode, k)
+            ix.set_path(True)
+            s2, i2 = ix.search(q, k, mask_words=words)
+            ix.set_path(False)
+            assert np.array_equal(i2, i) and bits_equal(s2, s)
+    assert ix.overflow_redos() == 0
+    ix.close()
+
+
+def test_candidate_overflow_is_redone_exactly(T, oracle):
+    """An index ordered against the sampler: every block the sampling pass reads
+    holds poor matches and all the others hold near-duplicates of the query, so
+    the floor is low, the candidate buffer overflows, and the query is redone
+    through the full list path with the same exact answer."""
+    O = oracle
+    dim, bits, n = 64, 4, 64 * 32 * 24
+    rng = np.random.default_rng(8)
+    q = unit_gaussian(3, dim, seed=9)
+    v = -np.tile(q[0], (n, 1)) + 0.3 * rng.standard_normal((n, dim)).astype(np.float32)   # poor matches
+    block = np.arange(n) // 32
+    good = block % 4 != 0                           # k=10 -> the sampler reads every 64th block (a multiple of 4)
+    v[good] = np.tile(q[0], (int(good.sum()), 1)) + 0.3 * rng.standard_normal((int(good.sum()), dim)).astype(np.float32)
+    oidx = OracleIndex(O, dim, bits, v.astype(np.float32))
+    ix = to_native(T, oidx)
+    s, i = ix.search(q, 10)
+    os_, oi = oidx.search(q, 10)
+    assert np.array_equal(i, oi) and bits_equal(s, os_)
+    assert ix.overflow_redos() >= 1
+    ix.close()
+
+
+def test_all_equal_scores(T, oracle):
+    """Every row identical: all scores tie bitwise, far more ties than the
+    candidate buffer holds; the lowest slots must come back."""
+    O = oracle
+    dim, bits, n = 64, 4, 50_000
+    row = unit_gaussian(1, dim, seed=3)
+    oidx = OracleIndex(O, dim, bits, np.tile(row, (n, 1)))
+    ix = to_native(T, oidx)
+    q = unit_gaussian(2, dim, seed=4)
+    for k in (10, 100):
+        s, i = ix.search(q, k)
+        assert np.array_equal(i, np.tile(np.arange(k), (2, 1)))
+        os_, oi = oidx.search(q, k)
+        assert np.array_equal(i, oi) and bits_equal(s, os_)
+    ix.close()

@@ -30,7 +30,7 @@ EXPORTS = [
     "tv_index_upload_seq_dev", "tv_index_append_rows", "tv_index_swap_remove", "tv_index_download_seq", "tv_index_len", "tv_index_dim",
     "tv_index_bits", "tv_validate_queries", "tv_pack_mask", "tv_search", "tv_search_dev", "tv_debug_scan",
     "tv_debug_prepare", "tv_last_scan_ms", "tv_index_device_ptrs", "tv_host_rotation_tables", "tv_host_codebook",
-    "tv_debug_stream_probe",
+    "tv_debug_stream_probe", "tv_debug_set_path", "tv_debug_overflow_redos",
 ]
 
 _lib = None
@@ -79,6 +79,8 @@ def lib():
     L.tv_debug_prepare.argtypes = [vp, vp, sz, vp, vp, vp]
     L.tv_last_scan_ms.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(i32)]
     L.tv_index_device_ptrs.argtypes = [vp, C.POINTER(vp), C.POINTER(vp), C.POINTER(sz)]
+    L.tv_debug_set_path.argtypes = [vp, i32]
+    L.tv_debug_overflow_redos.argtypes = [vp, C.POINTER(sz)]
     L.tv_debug_stream_probe.argtypes = [vp, vp, vp, sz, i32, C.POINTER(C.c_float)]
     L.tv_host_rotation_tables.argtypes = [i32, vp, vp, C.POINTER(i32), C.POINTER(C.c_float)]
     L.tv_host_codebook.argtypes = [i32, i32, vp, vp]
@@ -214,6 +216,14 @@ class NativeIndex:
         n = C.c_int(0)
         check(lib().tv_last_scan_ms(self.h, C.byref(ms), C.byref(n)))
         return ms.value, n.value
+
+    def set_path(self, force_full_lists):
+        check(lib().tv_debug_set_path(self.h, int(bool(force_full_lists))))
+
+    def overflow_redos(self):
+        c = C.c_size_t(0)
+        check(lib().tv_debug_overflow_redos(self.h, C.byref(c)))
+        return c.value
 
     def stream_probe(self, d_src_ptr, d_dst_ptr, nbytes, reps=5):
         """Mean ms per launch of a read-sum (d_dst_ptr None) or copy kernel over nbytes."""

@@ -7,6 +7,7 @@
 #include <cstring>
 #include <new>
 #include <string>
+#include <vector>
 
 #include "tv_internal.h"
 
@@ -170,9 +171,10 @@ void fill_scan_args(const tv_index *ix, tv::ScanArgs &a) {
     a.nch = ix->geo.nch;
     std::memcpy(a.lv, ix->levels, 16);
     a.classic = effective_mode(ix) == TV_SCORE_L_CLASSIC;
+    a.b_step = 1;
 }
 
-constexpr size_t kChunkQueries = 4096;
+constexpr size_t kChunkQueries = 1024;
 constexpr int kMaxTimedTiles = int(kChunkQueries / tv::kQTile);
 
 struct EventPool {
@@ -192,29 +194,23 @@ int ensure_events() {
     return TV_OK;
 }
 
-// The seam: search::search over device-resident inputs and outputs.
-int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, const uint64_t *d_mask,
-                  size_t n_allowed, float *d_out_scores, int64_t *d_out_idx, size_t *out_k_eff) {
+// Full-range search without sampling: per-lane lists with shared thresholds for
+// k <= 32, dense scores + radix select beyond.  Always exact; used for the
+// queries whose candidate buffer overflowed and for very large k.
+int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff, const uint64_t *d_mask,
+                  float *d_out_scores, int64_t *d_out_idx, bool timed_run) {
     const size_t n = ix->n;
-    size_t k_eff = std::min(std::min(k, n), n_allowed);  // lib.rs:1460, search.rs:3222-3225
-    if (out_k_eff) *out_k_eff = k_eff;
-    ix->last_scan_ms = 0.0f;
-    ix->last_scan_launches = 0;
-    if (k_eff == 0 || nq == 0) return TV_OK;                // search.rs:3226-3229
-    if (n >= (size_t(1) << 31)) { g_last_error = "index too large for 31-bit slots"; return TV_ERR_BAD_ARGUMENT; }
     const tv::Geometry &g = ix->geo;
     const int mode = effective_mode(ix);
-    if (mode == TV_SCORE_P && g.bits != 4) { g_last_error = "score mode P needs 4-bit codes"; return TV_ERR_BAD_ARGUMENT; }
     const bool mode_p = mode == TV_SCORE_P;
     const bool lists = k_eff <= size_t(tv::kMaxListK);
-    int rc = ensure_events();
-    if (rc != TV_OK) return rc;
-
+    int rc = TV_OK;
     for (size_t q0 = 0; q0 < nq; q0 += kChunkQueries) {
         const size_t cq = std::min(kChunkQueries, nq - q0);
-        const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_tile_queries(g.nch, lists ? int(k_eff) : 1));
+        const int kl = lists ? int(k_eff) : 1;
+        const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_tile_queries(g.nch, kl));
         const size_t n_tiles = (cq + tile_q - 1) / tile_q;
-        const int grid = tv::scan_grid_blocks(ix->device, mode_p, g.nch, lists ? int(k_eff) : 1, int(tile_q));
+        const int grid = tv::scan_grid_blocks(ix->device, mode_p, g.nch, kl, int(tile_q));
         const size_t total_threads = size_t(grid) * tv::kScanThreads;
         size_t need = prepare_bytes(ix, cq) + round_up(n_tiles * tv::kQTile * 4, 256);
         if (lists) need += 2 * round_up(k_eff * total_threads * 4, 256) + round_up(total_threads * 4, 256);
@@ -250,33 +246,172 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             a.qscale = pq.d_qscale + t * tile_q;
             a.qbias = pq.d_qbias + t * tile_q;
             a.nq_tile = int(std::min<size_t>(tile_q, cq - t * tile_q));
-            a.k = int(lists ? k_eff : 1);
+            a.k = kl;
             a.gtau = d_tau + t * tv::kQTile;
             a.part_scores = d_part_s; a.part_idx = d_part_i; a.part_cnt = d_part_c;
             a.score_out = d_dense;
-            if (!lists && d_mask) // blocks without an allowed slot are skipped by the scan: mark them excluded
+            a.share_tau = 1;
+            if (!lists && d_mask)  // blocks without an allowed slot are skipped by the scan: mark them excluded
                 TV_HIP(tv::launch_fill_i32(reinterpret_cast<int *>(d_dense), 0x7fc00000, size_t(a.nq_tile) * n, ix->stream));
-            const bool timed = int(t) < kMaxTimedTiles;
+            const bool timed = timed_run && int(t) < kMaxTimedTiles;
+            const int smode = lists ? tv::kModeLists : tv::kModeDump;
             if (timed) TV_HIP(hipEventRecord(g_events.start[t], ix->stream));
-            if (mode_p) TV_HIP(tv::launch_scan_p4(a, grid, !lists, ix->stream));
-            else TV_HIP(tv::launch_scan_lut(a, grid, !lists, ix->stream));
+            if (mode_p) TV_HIP(tv::launch_scan_p4(a, grid, smode, ix->stream));
+            else TV_HIP(tv::launch_scan_lut(a, grid, smode, ix->stream));
             if (timed) TV_HIP(hipEventRecord(g_events.stop[t], ix->stream));
             float *os = d_out_scores + (q0 + t * tile_q) * k_eff;
             int64_t *oi = d_out_idx + (q0 + t * tile_q) * k_eff;
             if (lists) {
-                const int qmod = mode_p ? tv::kQTile : tv::lut_launch_ql(g.nch, int(k_eff), a.nq_tile);
+                const int qmod = mode_p ? tv::kQTile : tv::lut_launch_ql(g.nch, kl, a.nq_tile);
                 TV_HIP(tv::launch_merge(d_part_s, d_part_i, d_part_c, int(total_threads), qmod, int(k_eff), int(k_eff),
-                                        a.nq_tile, os, oi, ix->stream));
+                                        a.nq_tile, os, oi, nullptr, ix->stream));
             } else {
                 TV_HIP(tv::launch_select_topk(d_dense, n, a.nq_tile, k_eff, d_keys, d_hist, os, oi, ix->stream));
             }
         }
+        TV_HIP(hipStreamSynchronize(ix->stream));
+        for (size_t t = 0; timed_run && t < n_tiles && int(t) < kMaxTimedTiles; ++t) {
+            float ms = 0.0f;
+            TV_HIP(hipEventElapsedTime(&ms, g_events.start[t], g_events.stop[t]));
+            ix->last_scan_ms += ms;
+            ix->last_scan_launches += 1;
+        }
+    }
+    return TV_OK;
+}
+
+// Sampling plan of a search: block strides of the successive append-mode scans,
+// the last one being 1 (the full scan).  Sizes shrink from the full index by
+// the factor target/k_floor per level until a level is small enough for all of
+// its slots to be appended; each later level, filtered by the floor of the one
+// before, then appends about `target` candidates per query, and the sampling
+// levels together read only about k_floor/target of the index.
+std::vector<uint32_t> sampling_steps(size_t n_blocks, size_t k_floor) {
+    const double n_slots = double(n_blocks * tv::kVecBlock);
+    const double target = double(std::max<size_t>(1024, 4 * k_floor));
+    const double ratio = target / double(k_floor);
+    std::vector<uint32_t> steps;
+    std::vector<double> sizes;
+    for (double sample = n_slots / ratio; ; sample /= ratio) {
+        sizes.push_back(sample);
+        if (sample <= target) break;
+    }
+    if (n_slots > target) {
+        for (size_t i = sizes.size(); i-- > 0;) {
+            const size_t sample_blocks = std::max<size_t>(1, size_t(sizes[i]) / tv::kVecBlock);
+            const size_t step = n_blocks / sample_blocks;
+            if (step > 1 && (steps.empty() || step < steps.back())) steps.push_back(uint32_t(step));
+        }
+    }
+    steps.push_back(1);
+    return steps;
+}
+
+// The seam: search::search over device-resident inputs and outputs.
+//
+// Sample-then-filter.  Scans run in append mode: every allowed slot whose score
+// reaches the query's floor is appended to a small per-query buffer, and a sort
+// of that buffer yields either the next floor (sampling levels) or the answer
+// (the full scan).  A floor is the k-th best score among slots actually
+// scanned, hence a lower bound of the true k-th best, so the full scan appends
+// every member of the true top-k; ties at the floor are kept (>=) and resolved
+// by the same total order as everywhere else.
+int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, const uint64_t *d_mask,
+                  size_t n_allowed, float *d_out_scores, int64_t *d_out_idx, size_t *out_k_eff) {
+    const size_t n = ix->n;
+    size_t k_eff = std::min(std::min(k, n), n_allowed);  // lib.rs:1460, search.rs:3222-3225
+    if (out_k_eff) *out_k_eff = k_eff;
+    ix->last_scan_ms = 0.0f;
+    ix->last_scan_launches = 0;
+    if (k_eff == 0 || nq == 0) return TV_OK;                // search.rs:3226-3229
+    if (n >= (size_t(1) << 31)) { g_last_error = "index too large for 31-bit slots"; return TV_ERR_BAD_ARGUMENT; }
+    const tv::Geometry &g = ix->geo;
+    const int mode = effective_mode(ix);
+    if (mode == TV_SCORE_P && g.bits != 4) { g_last_error = "score mode P needs 4-bit codes"; return TV_ERR_BAD_ARGUMENT; }
+    const bool mode_p = mode == TV_SCORE_P;
+    int rc = ensure_events();
+    if (rc != TV_OK) return rc;
+    if (k_eff > size_t(tv::kMaxSampledK) || ix->force_robust)
+        return search_robust(ix, d_queries, nq, k_eff, d_mask, d_out_scores, d_out_idx, true);
+
+    const size_t n_blocks = (n + tv::kVecBlock - 1) / tv::kVecBlock;
+    // sampling levels take the k_floor-th best as the floor: a deeper order statistic is steadier
+    const size_t k_floor = std::max<size_t>(k_eff, 16);
+    const std::vector<uint32_t> steps = sampling_steps(n_blocks, k_floor);
+    std::vector<uint32_t> h_over;
+
+    for (size_t q0 = 0; q0 < nq; q0 += kChunkQueries) {
+        const size_t cq = std::min(kChunkQueries, nq - q0);
+        const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_tile_queries(g.nch, 1));
+        const size_t n_tiles = (cq + tile_q - 1) / tile_q;
+        const size_t cq_pad = n_tiles * tile_q;
+        const int grid = tv::scan_grid_blocks(ix->device, mode_p, g.nch, 0, int(tile_q));
+        const size_t seg_stride = size_t(grid);
+        size_t need = prepare_bytes(ix, cq) + round_up(n_tiles * tv::kQTile * 4, 256) +
+                      round_up(cq_pad * seg_stride * tv::kSegCap * 8, 256) + round_up(cq_pad * seg_stride * 4, 256) +
+                      round_up(cq_pad * 4, 256);
+        rc = ensure_workspace(ix, need + 65536);
+        if (rc != TV_OK) return rc;
+        Arena ar;
+        ar.base = static_cast<uint8_t *>(ix->ws);
+        Prepared pq;
+        rc = prepare_queries(ix, ar, d_queries + q0 * g.dim, cq, pq);
+        if (rc != TV_OK) return rc;
+        int *d_tau = ar.take<int>(n_tiles * tv::kQTile);
+        uint64_t *d_cand = ar.take<uint64_t>(cq_pad * seg_stride * tv::kSegCap);
+        uint32_t *d_cnt = ar.take<uint32_t>(cq_pad * seg_stride);
+        uint32_t *d_over = ar.take<uint32_t>(cq_pad);
+        TV_HIP(tv::launch_fill_i32(d_tau, int(0x807fffffu) /* order key of -inf */, n_tiles * tv::kQTile, ix->stream));
+        TV_HIP(tv::launch_fill_i32(reinterpret_cast<int *>(d_over), 0, cq_pad, ix->stream));
+
+        for (size_t lv = 0; lv < steps.size(); ++lv) {
+            const bool last = lv + 1 == steps.size();
+            const size_t level_blocks = (n_blocks + steps[lv] - 1) / steps[lv];
+            // level 1 appends every slot it reads: two blocks per workgroup fill a segment exactly
+            const int lgrid = int(std::min<size_t>(size_t(grid), std::max<size_t>(1, (level_blocks + 1) / 2)));
+            for (size_t t = 0; t < n_tiles; ++t) {
+                tv::ScanArgs a;
+                fill_scan_args(ix, a);
+                a.mask = d_mask;
+                a.tables = pq.d_tables + t * (mode_p ? pq.table_bytes_per_tile : tile_q * size_t(g.nch) * 1024);
+                a.qscale = pq.d_qscale + t * tile_q;
+                a.qbias = pq.d_qbias + t * tile_q;
+                a.nq_tile = int(std::min<size_t>(tile_q, cq - t * tile_q));
+                a.k = 1;
+                a.gtau = d_tau + t * tv::kQTile;
+                a.b_step = steps[lv];
+                a.cand = d_cand + t * tile_q * seg_stride * tv::kSegCap;
+                a.cand_cnt = d_cnt + t * tile_q * seg_stride;
+                a.seg_stride = uint32_t(seg_stride);
+                const bool timed = last && int(t) < kMaxTimedTiles;
+                if (timed) TV_HIP(hipEventRecord(g_events.start[t], ix->stream));
+                if (mode_p) TV_HIP(tv::launch_scan_p4(a, lgrid, tv::kModeAppend, ix->stream));
+                else TV_HIP(tv::launch_scan_lut(a, lgrid, tv::kModeAppend, ix->stream));
+                if (timed) TV_HIP(hipEventRecord(g_events.stop[t], ix->stream));
+            }
+            TV_HIP(tv::launch_final(d_cand, d_cnt, uint32_t(lgrid), uint32_t(seg_stride), int(k_eff), int(k_floor),
+                                    int(cq), d_out_scores + q0 * k_eff, d_out_idx + q0 * k_eff, d_over,
+                                    last ? nullptr : d_tau, int(tile_q), ix->stream));
+        }
+        h_over.resize(cq);
+        TV_HIP(hipMemcpyAsync(h_over.data(), d_over, cq * sizeof(uint32_t), hipMemcpyDeviceToHost, ix->stream));
         TV_HIP(hipStreamSynchronize(ix->stream));
         for (size_t t = 0; t < n_tiles && int(t) < kMaxTimedTiles; ++t) {
             float ms = 0.0f;
             TV_HIP(hipEventElapsedTime(&ms, g_events.start[t], g_events.stop[t]));
             ix->last_scan_ms += ms;
             ix->last_scan_launches += 1;
+        }
+        // queries whose candidates did not fit (an unlucky sample, adversarial order): redo exactly
+        for (size_t qa = 0; qa < cq;) {
+            if (!h_over[qa]) { ++qa; continue; }
+            size_t qb = qa;
+            while (qb < cq && h_over[qb]) ++qb;
+            ix->overflow_redos += qb - qa;
+            rc = search_robust(ix, d_queries + (q0 + qa) * g.dim, qb - qa, k_eff, d_mask,
+                               d_out_scores + (q0 + qa) * k_eff, d_out_idx + (q0 + qa) * k_eff, false);
+            if (rc != TV_OK) return rc;
+            qa = qb;
         }
     }
     return TV_OK;
@@ -655,8 +790,8 @@ int tv_debug_scan(tv_index *ix, const float *queries, size_t nq, int32_t *acc_ou
         a.acc_out = d_acc;
         a.score_out = d_sc;
         const int grid = tv::scan_grid_blocks(ix->device, mode_p, g.nch, 1, int(tile_q));
-        if (mode_p) TV_HIP(tv::launch_scan_p4(a, grid, true, ix->stream));
-        else TV_HIP(tv::launch_scan_lut(a, grid, true, ix->stream));
+        if (mode_p) TV_HIP(tv::launch_scan_p4(a, grid, tv::kModeDump, ix->stream));
+        else TV_HIP(tv::launch_scan_lut(a, grid, tv::kModeDump, ix->stream));
         if (acc_out) TV_HIP(hipMemcpyAsync(acc_out + q0 * n, d_acc, cq * n * 4, hipMemcpyDeviceToHost, ix->stream));
         if (scores_out) TV_HIP(hipMemcpyAsync(scores_out + q0 * n, d_sc, cq * n * 4, hipMemcpyDeviceToHost, ix->stream));
         TV_HIP(hipStreamSynchronize(ix->stream));
@@ -722,6 +857,18 @@ int tv_debug_stream_probe(tv_index *ix, const void *d_src, void *d_dst, size_t b
     float ms = 0.0f;
     TV_HIP(hipEventElapsedTime(&ms, g_events.start[0], g_events.stop[0]));
     if (ms_per_rep) *ms_per_rep = ms / float(reps);
+    return TV_OK;
+}
+
+int tv_debug_set_path(tv_index *ix, int force_full_lists) {
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    ix->force_robust = force_full_lists != 0;
+    return TV_OK;
+}
+
+int tv_debug_overflow_redos(const tv_index *ix, size_t *count) {
+    if (!ix || !count) return TV_ERR_BAD_ARGUMENT;
+    *count = ix->overflow_redos;
     return TV_OK;
 }
 

@@ -16,6 +16,15 @@ constexpr int kChunkGroups = 32; // byte-groups per native chunk
 constexpr int kQTile = 32;       // queries per MFMA column tile
 constexpr int kScanThreads = 256;
 constexpr int kMaxListK = 32;    // largest k served by the per-lane lists
+constexpr int kSegCap = 64;      // candidate keys one workgroup may append per query and launch
+constexpr int kFinalCap = 8192;  // candidate keys per query the final sort holds (64 KiB of LDS)
+constexpr int kMaxSampledK = 512;   // largest k served by sample-then-filter
+
+// What a scan launch does with the scores it computes.
+enum { kModeLists = 0,   // per-lane top-k lists (written out for k_merge)
+       kModeDump = 1,    // every score (and accumulator) to dense rows
+       kModeAppend = 2   // every allowed slot scoring >= the query's fixed floor to a candidate buffer
+};
 
 // Native device layout of the codes ("vm32"): the byte of (block b, group g,
 // vector i) lives at ((b*nch + g/32)*64 + ((g%32)/16)*32 + i)*16 + g%16, groups
@@ -50,6 +59,11 @@ struct ScanArgs {
     int32_t *acc_out;          // dump mode: [nq_tile][n] (may be null)
     float *score_out;          // dump mode: [nq_tile][n]
     int classic;               // mode L: 1 = fma flush per 256 groups, 0 = u32 epilogue
+    uint32_t b_step;           // 1, or a sampling stride: only blocks j*b_step are scanned
+    int share_tau;             // lists mode: waves share and raise gtau while scanning
+    uint64_t *cand;            // append mode: [nq_tile][seg_stride][kSegCap] sort keys, one segment per workgroup
+    uint32_t *cand_cnt;        // append mode: [nq_tile][seg_stride] counts (above kSegCap: that segment overflowed)
+    uint32_t seg_stride;       // segments allocated per query (>= grid of the launch)
 };
 
 // ---- launchers (tv_kernels.hip) ----
@@ -79,11 +93,20 @@ size_t scan_lds_bytes(int mode_p, int nch, int k, int lut_queries);
 int lut_tile_queries(int nch, int k);
 // Queries per LDS entry (1, 2 or 4) the LUT scan launch picks for nq_tile queries.
 int lut_launch_ql(int nch, int k, int nq_tile);
-hipError_t launch_scan_p4(const ScanArgs &a, int grid, bool dump, hipStream_t s);
-hipError_t launch_scan_lut(const ScanArgs &a, int grid, bool dump, hipStream_t s);
+hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s);
+hipError_t launch_scan_lut(const ScanArgs &a, int grid, int mode, hipStream_t s);
+// out_tau == nullptr: write the k_eff best of the merged lists; else write only the
+// order key of the k_eff-th best (a floor at least k_eff scanned slots reach) per query.
 hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, const int *part_cnt, int total_threads,
                         int qmod, int k, int k_eff, int nq_tile, float *out_scores, int64_t *out_idx,
-                        hipStream_t s);
+                        int *out_tau, hipStream_t s);
+// Gathers each query's candidate segments (n_seg of them, seg_stride allocated), sorts, and either
+// emits the k_eff best (tau_out == nullptr; a query that did not fit is flagged in overflow) or, for a
+// sampling level, writes the order key of the k_floor-th best as the query's next floor to
+// tau_out[(q / tau_stride_q) * kQTile + q % tau_stride_q].
+hipError_t launch_final(const uint64_t *cand, const uint32_t *cand_cnt, uint32_t n_seg, uint32_t seg_stride,
+                        int k_eff, int k_floor, int nq, float *out_scores, int64_t *out_idx, uint32_t *overflow,
+                        int *tau_out, int tau_stride_q, hipStream_t s);
 hipError_t launch_fill_i32(int *p, int v, size_t n, hipStream_t s);
 hipError_t launch_probe(const void *src, void *dst, size_t bytes, int copy, uint32_t *sink, hipStream_t s);
 // Exact top-k of a dense score row per query (NaN = excluded slot).
@@ -122,4 +145,6 @@ struct tv_index {
     size_t ws_bytes = 0;
     float last_scan_ms = 0.0f;
     int last_scan_launches = 0;
+    int force_robust = 0;          // test hook: skip sample-then-filter
+    size_t overflow_redos = 0;     // queries redone because their candidate buffer overflowed
 };

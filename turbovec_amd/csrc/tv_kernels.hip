@@ -321,15 +321,17 @@ __device__ __forceinline__ uint32_t levels_of(uint32_t nib, uint32_t t0, uint32_
     return __builtin_amdgcn_perm(t1, t0, selA) & __builtin_amdgcn_perm(t3, t2, selB);
 }
 
-template <int U, bool DUMP, bool W_LDS>
+template <int U, int MODE, bool W_LDS>
 __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
+    constexpr bool LISTS = MODE == kModeLists, DUMP = MODE == kModeDump, APPEND = MODE == kModeAppend;
     const int nch = a.nch, k = a.k;
     uint8_t *sW = smem;
     const size_t w_bytes = W_LDS ? size_t(nch) * 2048 : 0;
     float *ls = reinterpret_cast<float *>(smem + w_bytes);
-    uint32_t *li = reinterpret_cast<uint32_t *>(ls + (DUMP ? 0 : k * kScanThreads));
-    int *stau = reinterpret_cast<int *>(li + (DUMP ? 0 : k * kScanThreads));
+    uint32_t *li = reinterpret_cast<uint32_t *>(ls + (LISTS ? k * kScanThreads : 0));
+    int *stau = reinterpret_cast<int *>(li + (LISTS ? k * kScanThreads : 0));
+    uint32_t *scnt = reinterpret_cast<uint32_t *>(stau);  // append mode: candidates per query of this workgroup
 
     const int tid = threadIdx.x;
     if (W_LDS) {
@@ -337,7 +339,8 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
         uint4 *dst = reinterpret_cast<uint4 *>(sW);
         for (int i = tid; i < nch * 128; i += kScanThreads) dst[i] = src[i];
     }
-    if (!DUMP && tid < kQTile) stau[tid] = a.gtau[tid];
+    if (LISTS && tid < kQTile) stau[tid] = a.gtau[tid];
+    if (APPEND && tid < kQTile) scnt[tid] = 0u;
     __syncthreads();
 
     const int lane = tid & 63, wave = tid >> 6;
@@ -346,12 +349,18 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
     const float qs = active ? a.qscale[qn] : 0.0f;
     const float qb = active ? a.qbias[qn] : 0.0f;
     const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
+    // append mode: a fixed per-query floor; NaN for idle lanes so no compare passes
+    const float tau_fixed = APPEND ? (active ? order_unkey(a.gtau[qn]) : __int_as_float(0x7fc00000)) : 0.0f;
 
+    // Logical blocks j = 0..nj-1 stand for physical blocks j*step (step > 1 samples the index).
+    const uint32_t step = a.b_step;
+    const uint32_t nj = (a.n_blocks + step - 1) / step;
     const uint32_t total_waves = gridDim.x * (kScanThreads / 64);
-    const uint32_t gw = blockIdx.x * (kScanThreads / 64) + wave;
-    const uint32_t per = (a.n_blocks + total_waves - 1) / total_waves;
-    const uint32_t b_begin = min(gw * per, a.n_blocks);
-    const uint32_t b_end = min(b_begin + per, a.n_blocks);
+    const uint32_t gw = wave * gridDim.x + blockIdx.x;  // consecutive blocks go to different workgroups
+    // Blocks are dealt round-robin to the waves of the grid: wave gw takes logical blocks gw,
+    // gw + total_waves, ...  Neighbouring rows (clustered data, contiguous allowlists) then spread
+    // over all workgroups instead of piling into one.
+    const uint32_t j_begin = gw, j_end = nj;
 
     LaneList L{0, 0.0f, 0u, 0};
     const uint4 *codes = reinterpret_cast<const uint4 *>(a.codes) + lane;
@@ -359,24 +368,26 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
     const uint4 *wlds = reinterpret_cast<const uint4 *>(sW) + lane;
 
     // first block with at least one allowed slot (search.rs:3015-3029)
-    auto live_from = [&](uint32_t b) -> uint32_t {
-        if (a.mask == nullptr) return b;
-        while (b < b_end) {
+    auto live_from = [&](uint32_t j) -> uint32_t {
+        if (a.mask == nullptr) return j;
+        while (j < j_end) {
+            const uint32_t b = j * step;
             const uint64_t w = a.mask[b >> 1];
             if (uint32_t(w >> ((b & 1) * 32)) != 0u) break;
-            ++b;
+            j += total_waves;
         }
-        return b;
+        return j;
     };
 
-    uint32_t b = live_from(b_begin);
+    uint32_t j = live_from(j_begin);
     uint4 buf[U];
-    if (b < b_end) {
+    if (j < j_end) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(b) * nch + u) * 64];
+        for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(j) * step * nch + u) * 64];
     }
-    while (b < b_end) {
-        const uint32_t nb = live_from(b + 1);
+    while (j < j_end) {
+        const uint32_t nj_live = live_from(j + total_waves);
+        const uint32_t b = j * step;
         v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         for (int c0 = 0; c0 < nch; c0 += U) {
             uint4 cur[U];
@@ -385,9 +396,9 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
             if (c0 + U < nch) {
 #pragma unroll
                 for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(b) * nch + c0 + U + u) * 64];
-            } else if (nb < b_end) {
+            } else if (nj_live < j_end) {
 #pragma unroll
-                for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(nb) * nch + u) * 64];
+                for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(nj_live) * step * nch + u) * 64];
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
@@ -433,8 +444,22 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
                     }
                 }
             }
+        } else if (APPEND) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float s = fmaf(float(acc[r]), qs, qb) * vs[r];
+                if (s >= tau_fixed) {
+                    const int i = 8 * (r >> 2) + 4 * h + (r & 3);
+                    const uint32_t slot = slot0 + i;
+                    if (slot < a.n && ((mw >> i) & 1u)) {
+                        const uint32_t pos = atomicAdd(&scnt[qn], 1u);
+                        if (pos < kSegCap)
+                            a.cand[(size_t(qn) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(s, slot);
+                    }
+                }
+            }
         } else {
-            if ((b & 3u) == 0u && lane < kQTile) atomicMax(&stau[lane], a.gtau[lane]);
+            if (a.share_tau && (j & 3u) == 0u && lane < kQTile) atomicMax(&stau[lane], a.gtau[lane]);
             const float tau = order_unkey(stau[qn]);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -443,7 +468,7 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
                 const float s = fmaf(float(acc[r]), qs, qb) * vs[r];
                 if (active && s >= tau && (L.cnt < k || ranks_before(s, slot, L.worst_s, L.worst_i))) {
                     if (slot < a.n && ((mw >> i) & 1u)) {
-                        if (list_offer(L, ls, li, kScanThreads, tid, k, s, slot)) {
+                        if (list_offer(L, ls, li, kScanThreads, tid, k, s, slot) && a.share_tau) {
                             const int key = order_key(L.worst_s);
                             if (atomicMax(&stau[qn], key) < key) atomicMax(&a.gtau[qn], key);
                         }
@@ -451,10 +476,10 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
                 }
             }
         }
-        b = nb;
+        j = nj_live;
     }
 
-    if (!DUMP) {
+    if (LISTS) {
         const size_t total_threads = size_t(gridDim.x) * kScanThreads;
         const size_t gt = size_t(blockIdx.x) * kScanThreads + tid;
         a.part_cnt[gt] = L.cnt;
@@ -462,6 +487,10 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
             a.part_scores[size_t(e) * total_threads + gt] = ls[e * kScanThreads + tid];
             a.part_idx[size_t(e) * total_threads + gt] = li[e * kScanThreads + tid];
         }
+    }
+    if (APPEND) {
+        __syncthreads();
+        if (tid < a.nq_tile) a.cand_cnt[size_t(tid) * a.seg_stride + blockIdx.x] = scnt[tid];
     }
 }
 
@@ -475,7 +504,7 @@ __global__ __launch_bounds__(256) void k_merge(const float *__restrict__ part_sc
                                                const uint32_t *__restrict__ part_idx,
                                                const int *__restrict__ part_cnt, int total_threads, int qmod,
                                                int k, int k_eff, int sort_n, float *__restrict__ out_scores,
-                                               int64_t *__restrict__ out_idx) {
+                                               int64_t *__restrict__ out_idx, int *__restrict__ out_tau) {
     extern __shared__ __align__(16) uint8_t msm[];
     float *ls = reinterpret_cast<float *>(msm);
     uint32_t *li = reinterpret_cast<uint32_t *>(ls + k * 256);
@@ -513,11 +542,115 @@ __global__ __launch_bounds__(256) void k_merge(const float *__restrict__ part_sc
             __syncthreads();
         }
     }
+    if (out_tau != nullptr) {
+        // sampling pass: publish a floor that at least k_eff scanned slots reach
+        if (t == 0) {
+            float s = 0.0f; uint32_t idx = 0;
+            if (total >= k_eff && k_eff <= sort_n) sort_unkey(keys[k_eff - 1], s, idx);
+            out_tau[qn] = (total >= k_eff && k_eff <= sort_n) ? order_key(s == 0.0f ? -0.0f : s) : kTauInit;
+        }
+        return;
+    }
     for (int j = t; j < k_eff; j += 256) {
         float s; uint32_t idx;
         sort_unkey(keys[j], s, idx);
         out_scores[size_t(qn) * k_eff + j] = s;
         out_idx[size_t(qn) * k_eff + j] = int64_t(idx);
+    }
+}
+
+// ===========================================================================
+// Final selection over the candidates an append-mode scan collected: one
+// workgroup per query sorts its (few) candidate keys in LDS and emits the first
+// k_eff.  A query whose candidates did not fit is flagged for the caller to
+// redo through the list path.
+// ===========================================================================
+
+__global__ __launch_bounds__(256) void k_final(const uint64_t *__restrict__ cand,
+                                               const uint32_t *__restrict__ cand_cnt, uint32_t n_seg,
+                                               uint32_t seg_stride, int k_eff, int k_floor,
+                                               float *__restrict__ out_scores, int64_t *__restrict__ out_idx,
+                                               uint32_t *__restrict__ overflow, int *__restrict__ tau_out,
+                                               int tau_stride_q) {
+    __shared__ uint64_t keys[kFinalCap];
+    __shared__ uint32_t wave_sum[4];
+    __shared__ uint32_t any_full;
+    const int qn = blockIdx.x;
+    const int t = threadIdx.x;
+    const bool sampling = tau_out != nullptr;
+    int *tau_slot = sampling ? tau_out + (qn / tau_stride_q) * kQTile + qn % tau_stride_q : nullptr;
+    if (t == 0) any_full = 0u;
+    __syncthreads();
+    // every thread owns a contiguous run of this query's segments
+    const uint32_t per = (n_seg + 255) / 256;
+    const uint32_t s0 = min(uint32_t(t) * per, n_seg), s1 = min(s0 + per, n_seg);
+    const uint32_t *cnt = cand_cnt + size_t(qn) * seg_stride;
+    uint32_t mine = 0;
+    for (uint32_t sg = s0; sg < s1; ++sg) {
+        const uint32_t c = cnt[sg];
+        if (c > kSegCap) any_full = 1u;
+        mine += min(c, uint32_t(kSegCap));
+    }
+    // exclusive prefix over the 256 threads
+    uint32_t incl = mine;
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t v = __shfl_up(incl, off);
+        if ((t & 63) >= off) incl += v;
+    }
+    if ((t & 63) == 63) wave_sum[t >> 6] = incl;
+    __syncthreads();
+    uint32_t base = incl - mine, total = 0;
+    for (int w = 0; w < 4; ++w) { if (w < (t >> 6)) base += wave_sum[w]; total += wave_sum[w]; }
+    const bool too_many = total > uint32_t(kFinalCap);
+    if (!sampling && (too_many || any_full || total < uint32_t(k_eff))) {
+        if (t == 0) overflow[qn] = 1u;     // the caller redoes this query through the list path
+        return;
+    }
+    if (sampling && total < uint32_t(k_eff)) {
+        if (t == 0) *tau_slot = kTauInit;  // too few allowed slots sampled: the floor stays open
+        return;
+    }
+    // gather (a sampling level may keep any subset: dropping what does not fit only loosens the floor)
+    uint32_t pos = base;
+    for (uint32_t sg = s0; sg < s1; ++sg) {
+        const uint32_t c = min(cnt[sg], uint32_t(kSegCap));
+        const uint64_t *src = cand + (size_t(qn) * seg_stride + sg) * kSegCap;
+        for (uint32_t e = 0; e < c; ++e, ++pos)
+            if (pos < uint32_t(kFinalCap)) keys[pos] = src[e];
+    }
+    const uint32_t c_all = min(total, uint32_t(kFinalCap));
+    uint32_t sort_n = 2;
+    while (sort_n < c_all) sort_n <<= 1;
+    __syncthreads();
+    for (uint32_t i = c_all + t; i < sort_n; i += 256) keys[i] = 0ull;
+    __syncthreads();
+    for (uint32_t size = 2; size <= sort_n; size <<= 1) {
+        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+            for (uint32_t i = t; i < sort_n / 2; i += 256) {
+                const uint32_t lo = 2 * i - (i & (stride - 1));
+                const uint32_t hi = lo + stride;
+                const bool desc = (lo & size) == 0;
+                const uint64_t x = keys[lo], y = keys[hi];
+                if ((x < y) == desc) { keys[lo] = y; keys[hi] = x; }
+            }
+            __syncthreads();
+        }
+    }
+    if (sampling) {
+        if (t == 0) {
+            // the floor: the k_floor-th best sampled score (k_floor >= k_eff steadies the estimate)
+            const uint32_t pick = min(uint32_t(k_floor), c_all) - 1;
+            float s; uint32_t idx;
+            sort_unkey(keys[pick], s, idx);
+            *tau_slot = order_key(s == 0.0f ? -0.0f : s);
+        }
+        return;
+    }
+    for (int jj = t; jj < k_eff; jj += 256) {
+        float s; uint32_t idx;
+        sort_unkey(keys[jj], s, idx);
+        out_scores[size_t(qn) * k_eff + jj] = s;
+        out_idx[size_t(qn) * k_eff + jj] = int64_t(idx);
     }
 }
 
@@ -671,9 +804,9 @@ int scan_grid_blocks(int device, int mode_p, int nch, int k, int nq_tile) {
     return cus * per_cu;
 }
 
-hipError_t launch_scan_p4(const ScanArgs &a, int grid, bool dump, hipStream_t s) {
+hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s) {
     const size_t w = size_t(a.nch) * 2048;
-    const size_t lists = dump ? 64 : size_t(a.k) * kScanThreads * 8 + kQTile * sizeof(int);
+    const size_t lists = mode != kModeLists ? 64 : size_t(a.k) * kScanThreads * 8 + kQTile * sizeof(int);
     const bool w_lds = w + lists <= kLdsBudget;
     const size_t lds = (w_lds ? w : 0) + lists;
     hipError_t e = hipSuccess;
@@ -685,8 +818,9 @@ hipError_t launch_scan_p4(const ScanArgs &a, int grid, bool dump, hipStream_t s)
     } while (0)
 #define TV_PICK_P4(U)                                                                           \
     do {                                                                                        \
-        if (dump) { if (w_lds) TV_LAUNCH_P4(U, true, true); else TV_LAUNCH_P4(U, true, false); } \
-        else { if (w_lds) TV_LAUNCH_P4(U, false, true); else TV_LAUNCH_P4(U, false, false); }   \
+        if (mode == kModeDump) { if (w_lds) TV_LAUNCH_P4(U, kModeDump, true); else TV_LAUNCH_P4(U, kModeDump, false); } \
+        else if (mode == kModeAppend) { if (w_lds) TV_LAUNCH_P4(U, kModeAppend, true); else TV_LAUNCH_P4(U, kModeAppend, false); } \
+        else { if (w_lds) TV_LAUNCH_P4(U, kModeLists, true); else TV_LAUNCH_P4(U, kModeLists, false); } \
     } while (0)
     if (a.nch % 4 == 0) TV_PICK_P4(4);
     else if (a.nch % 2 == 0) TV_PICK_P4(2);
@@ -698,7 +832,7 @@ hipError_t launch_scan_p4(const ScanArgs &a, int grid, bool dump, hipStream_t s)
 
 hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, const int *part_cnt, int total_threads,
                         int qmod, int k, int k_eff, int nq_tile, float *out_scores, int64_t *out_idx,
-                        hipStream_t s) {
+                        int *out_tau, hipStream_t s) {
     if (nq_tile == 0 || k_eff == 0) return hipSuccess;
     int sort_n = 2;
     while (sort_n < 256 * k) sort_n <<= 1;
@@ -706,7 +840,16 @@ hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, cons
     hipError_t e = allow_lds(k_merge, lds);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(k_merge, dim3(nq_tile), dim3(256), lds, s, part_scores, part_idx, part_cnt, total_threads,
-                       qmod, k, k_eff, sort_n, out_scores, out_idx);
+                       qmod, k, k_eff, sort_n, out_scores, out_idx, out_tau);
+    return hipGetLastError();
+}
+
+hipError_t launch_final(const uint64_t *cand, const uint32_t *cand_cnt, uint32_t n_seg, uint32_t seg_stride,
+                        int k_eff, int k_floor, int nq, float *out_scores, int64_t *out_idx, uint32_t *overflow,
+                        int *tau_out, int tau_stride_q, hipStream_t s) {
+    if (nq == 0 || k_eff == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_final, dim3(nq), dim3(256), 0, s, cand, cand_cnt, n_seg, seg_stride, k_eff, k_floor,
+                       out_scores, out_idx, overflow, tau_out, tau_stride_q);
     return hipGetLastError();
 }
 

@@ -23,16 +23,17 @@ template <> struct LutWord<1> { typedef uint8_t type; };
 template <> struct LutWord<2> { typedef uint16_t type; };
 template <> struct LutWord<4> { typedef uint32_t type; };
 
-template <int QL, int U, bool DUMP, bool LUT_LDS>
+template <int QL, int U, int MODE, bool LUT_LDS>
 __global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
     typedef typename LutWord<QL>::type word_t;
+    constexpr bool LISTS = MODE == kModeLists, DUMP = MODE == kModeDump, APPEND = MODE == kModeAppend;
     extern __shared__ __align__(16) uint8_t smem[];
     const int nch = a.nch, k = a.k;
     const size_t lut_bytes = LUT_LDS ? size_t(nch) * 1024 * QL : 0;
     float *sct = reinterpret_cast<float *>(smem + lut_bytes);            // [4 waves][QL][32]
     float *ls = sct + 4 * QL * 32;
-    uint32_t *li = reinterpret_cast<uint32_t *>(ls + (DUMP ? 0 : k * kScanThreads));
-    int *stau = reinterpret_cast<int *>(li + (DUMP ? 0 : k * kScanThreads));
+    uint32_t *li = reinterpret_cast<uint32_t *>(ls + (LISTS ? k * kScanThreads : 0));
+    int *stau = reinterpret_cast<int *>(li + (LISTS ? k * kScanThreads : 0));
     const int tid = threadIdx.x;
 
     if (LUT_LDS) {
@@ -49,7 +50,9 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
             }
         }
     }
-    if (!DUMP && tid < kQTile) stau[tid] = tid < QL ? a.gtau[tid] : kTauInit;
+    if (LISTS && tid < kQTile) stau[tid] = tid < QL ? a.gtau[tid] : kTauInit;
+    uint32_t *scnt = reinterpret_cast<uint32_t *>(stau);  // append mode: candidates per query of this workgroup
+    if (APPEND && tid < kQTile) scnt[tid] = 0u;
     __syncthreads();
     const word_t *lut = LUT_LDS ? reinterpret_cast<const word_t *>(smem) : reinterpret_cast<const word_t *>(a.tables);
 
@@ -65,35 +68,38 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
     constexpr int per = QL * 32 >= 64 ? QL * 32 / 64 : 1;
     const int oq = lane % QL, vg = lane / QL;
     const bool owner = oq < a.nq_tile && vg * per < 32;
+    const float tau_fixed = APPEND ? (owner ? order_unkey(a.gtau[oq]) : __int_as_float(0x7fc00000)) : 0.0f;
 
+    const uint32_t step = a.b_step;
+    const uint32_t nj = (a.n_blocks + step - 1) / step;
     const uint32_t total_waves = gridDim.x * (kScanThreads / 64);
-    const uint32_t gw = blockIdx.x * (kScanThreads / 64) + wave;
-    const uint32_t per_wave = (a.n_blocks + total_waves - 1) / total_waves;
-    const uint32_t b_begin = min(gw * per_wave, a.n_blocks);
-    const uint32_t b_end = min(b_begin + per_wave, a.n_blocks);
+    const uint32_t gw = wave * gridDim.x + blockIdx.x;  // consecutive blocks go to different workgroups
+    const uint32_t j_begin = gw, j_end = nj;   // round-robin over the grid's waves
 
     LaneList L{0, 0.0f, 0u, 0};
     const uint4 *codes = reinterpret_cast<const uint4 *>(a.codes) + lane;
     float *my_sct = sct + wave * QL * 32;
 
-    auto live_from = [&](uint32_t b) -> uint32_t {
-        if (a.mask == nullptr) return b;
-        while (b < b_end) {
+    auto live_from = [&](uint32_t j) -> uint32_t {
+        if (a.mask == nullptr) return j;
+        while (j < j_end) {
+            const uint32_t b = j * step;
             const uint64_t w = a.mask[b >> 1];
             if (uint32_t(w >> ((b & 1) * 32)) != 0u) break;
-            ++b;
+            j += total_waves;
         }
-        return b;
+        return j;
     };
 
-    uint32_t b = live_from(b_begin);
+    uint32_t j = live_from(j_begin);
     uint4 buf[U];
-    if (b < b_end) {
+    if (j < j_end) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(b) * nch + u) * 64];
+        for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(j) * step * nch + u) * 64];
     }
-    while (b < b_end) {
-        const uint32_t nb = live_from(b + 1);
+    while (j < j_end) {
+        const uint32_t nj_live = live_from(j + total_waves);
+        const uint32_t b = j * step;
         uint32_t total[QL];
         float fa[QL];
 #pragma unroll
@@ -106,9 +112,9 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
             if (c0 + U < nch) {
 #pragma unroll
                 for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(b) * nch + c0 + U + u) * 64];
-            } else if (nb < b_end) {
+            } else if (nj_live < j_end) {
 #pragma unroll
-                for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(nb) * nch + u) * 64];
+                for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(nj_live) * step * nch + u) * 64];
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
@@ -173,19 +179,33 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
             }
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
             __builtin_amdgcn_wave_barrier();
-            if ((b & 3u) == 0u && lane < QL) atomicMax(&stau[lane], a.gtau[lane]);
-            if (owner) {
-                const float tau = order_unkey(stau[oq]);
+            if (APPEND) {
 #pragma unroll
                 for (int e = 0; e < per; ++e) {
-                    const int i = vg * per + e;
+                    const int i = (vg * per + e) & 31;
                     const float s = my_sct[oq * 32 + i];
                     const uint32_t slot = slot0 + i;
-                    if (s >= tau && (L.cnt < k || ranks_before(s, slot, L.worst_s, L.worst_i))) {
-                        if (slot < a.n && ((mw >> i) & 1u)) {
-                            if (list_offer(L, ls, li, kScanThreads, tid, k, s, slot)) {
-                                const int key = order_key(L.worst_s);
-                                if (atomicMax(&stau[oq], key) < key) atomicMax(&a.gtau[oq], key);
+                    if (s >= tau_fixed && slot < a.n && ((mw >> i) & 1u)) {
+                        const uint32_t pos = atomicAdd(&scnt[oq], 1u);
+                        if (pos < kSegCap)
+                            a.cand[(size_t(oq) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(s, slot);
+                    }
+                }
+            } else {
+                if (a.share_tau && (j & 3u) == 0u && lane < QL) atomicMax(&stau[lane], a.gtau[lane]);
+                if (owner) {
+                    const float tau = order_unkey(stau[oq]);
+#pragma unroll
+                    for (int e = 0; e < per; ++e) {
+                        const int i = vg * per + e;
+                        const float s = my_sct[oq * 32 + i];
+                        const uint32_t slot = slot0 + i;
+                        if (s >= tau && (L.cnt < k || ranks_before(s, slot, L.worst_s, L.worst_i))) {
+                            if (slot < a.n && ((mw >> i) & 1u)) {
+                                if (list_offer(L, ls, li, kScanThreads, tid, k, s, slot) && a.share_tau) {
+                                    const int key = order_key(L.worst_s);
+                                    if (atomicMax(&stau[oq], key) < key) atomicMax(&a.gtau[oq], key);
+                                }
                             }
                         }
                     }
@@ -194,10 +214,14 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
             __builtin_amdgcn_wave_barrier();
         }
-        b = nb;
+        j = nj_live;
     }
 
-    if (!DUMP) {
+    if (APPEND) {
+        __syncthreads();
+        if (tid < a.nq_tile) a.cand_cnt[size_t(tid) * a.seg_stride + blockIdx.x] = scnt[tid];
+    }
+    if (LISTS) {
         const size_t total_threads = size_t(gridDim.x) * kScanThreads;
         const size_t gt = size_t(blockIdx.x) * kScanThreads + tid;
         a.part_cnt[gt] = L.cnt;
@@ -210,8 +234,8 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
 
 static constexpr size_t kLdsBudgetL = 160 * 1024;
 
-static size_t lut_lds_bytes(int nch, int k, int ql, bool dump) {
-    const size_t lists = dump ? 0 : size_t(k) * kScanThreads * 8;
+static size_t lut_lds_bytes(int nch, int k, int ql, bool no_lists) {
+    const size_t lists = no_lists ? 0 : size_t(k) * kScanThreads * 8;
     return size_t(nch) * 1024 * ql + size_t(4) * ql * 32 * 4 + lists + kQTile * sizeof(int);
 }
 
@@ -235,8 +259,9 @@ int lut_launch_ql(int nch, int k, int nq_tile) {
 }
 
 // One launch serves a.nq_tile <= lut_tile_queries(nch, k) queries.
-hipError_t launch_scan_lut(const ScanArgs &a, int grid, bool dump, hipStream_t s) {
-    const int kk = dump ? 1 : a.k;
+hipError_t launch_scan_lut(const ScanArgs &a, int grid, int mode, hipStream_t s) {
+    const bool dump = mode != kModeLists;   // no list storage in LDS
+    const int kk = a.k;                     // the tile width is chosen for the list pass of the same search
     const int ql = lut_launch_ql(a.nch, kk, a.nq_tile);
     const bool in_lds = lut_lds_bytes(a.nch, kk, ql, dump) <= kLdsBudgetL;
     const size_t lds = in_lds ? lut_lds_bytes(a.nch, kk, ql, dump)
@@ -248,16 +273,21 @@ hipError_t launch_scan_lut(const ScanArgs &a, int grid, bool dump, hipStream_t s
         if (e != hipSuccess) return e;                                                           \
         hipLaunchKernelGGL((k_scan_lut<QL, U, D, W>), dim3(grid), dim3(kScanThreads), lds, s, a); \
     } while (0)
-#define TV_PICK_L(QL, U)                                                                         \
-    do { if (dump) TV_LAUNCH_L(QL, U, true, true); else TV_LAUNCH_L(QL, U, false, true); } while (0)
+#define TV_PICK_M(QL, U, W)                                                                      \
+    do {                                                                                         \
+        if (mode == kModeDump) TV_LAUNCH_L(QL, U, kModeDump, W);                                 \
+        else if (mode == kModeAppend) TV_LAUNCH_L(QL, U, kModeAppend, W);                        \
+        else TV_LAUNCH_L(QL, U, kModeLists, W);                                                  \
+    } while (0)
+#define TV_PICK_L(QL, U) TV_PICK_M(QL, U, true)
     const int u = a.nch % 2 == 0 ? 2 : 1;
     if (!in_lds) {
-        if (dump) { if (u == 2) TV_LAUNCH_L(1, 2, true, false); else TV_LAUNCH_L(1, 1, true, false); }
-        else { if (u == 2) TV_LAUNCH_L(1, 2, false, false); else TV_LAUNCH_L(1, 1, false, false); }
+        if (u == 2) TV_PICK_M(1, 2, false); else TV_PICK_M(1, 1, false);
     } else if (ql == 4) { if (u == 2) TV_PICK_L(4, 2); else TV_PICK_L(4, 1); }
     else if (ql == 2) { if (u == 2) TV_PICK_L(2, 2); else TV_PICK_L(2, 1); }
     else { if (u == 2) TV_PICK_L(1, 2); else TV_PICK_L(1, 1); }
 #undef TV_PICK_L
+#undef TV_PICK_M
 #undef TV_LAUNCH_L
     return hipGetLastError();
 }
