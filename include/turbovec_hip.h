@@ -143,9 +143,10 @@ int tv_debug_prepare(tv_index *ix, const float *queries, size_t nq,
  * tv_search* call on this index, measured with HIP events on its stream, and
  * how many launches that was. */
 int tv_last_scan_ms(const tv_index *ix, float *ms, int *launches);
-/* Path selection for tests: non-zero makes every search take the full-range
- * list / dense-select path instead of sample-then-filter (results must be
- * identical either way). */
+/* Path selection for tests (results must be identical either way): bit 0 makes
+ * every search take the full-range list / dense-select path instead of
+ * sample-then-filter; bit 1 keeps large batches on the one-tile-per-launch scan
+ * instead of the batched one. */
 int tv_debug_set_path(tv_index *ix, int force_full_lists);
 /* How many queries so far had to be redone through that path because their
  * candidate buffer overflowed. */

@@ -461,10 +461,11 @@ def test_sampled_path_matches_oracle_and_full_path(T, oracle, bits, mode):
             os_, oi = oidx.search(q, k, mask_words=words, mode=omode(O, mode))
             assert np.array_equal(i, oi), (mode, k)
             assert bits_equal(s, os_), (mode, k)
-            ix.set_path(True)
-            s2, i2 = ix.search(q, k, mask_words=words)
-            ix.set_path(False)
-            assert np.array_equal(i2, i) and bits_equal(s2, s)
+            for path in (1, 2):                   # full-range lists; one tile per launch
+                ix.set_path(path)
+                s2, i2 = ix.search(q, k, mask_words=words)
+                ix.set_path(0)
+                assert np.array_equal(i2, i) and bits_equal(s2, s)
     assert ix.overflow_redos() == 0
     ix.close()
 
@@ -505,4 +506,26 @@ def test_all_equal_scores(T, oracle):
         assert np.array_equal(i, np.tile(np.arange(k), (2, 1)))
         os_, oi = oidx.search(q, k)
         assert np.array_equal(i, oi) and bits_equal(s, os_)
+    ix.close()
+
+
+# ---- batched permute-dot scan (more than 32 queries per launch) ----
+@pytest.mark.parametrize("dim,n,nq", [(256, 40_003, 200), (1536, 20_011, 97), (512, 70_000, 129)])
+def test_batched_scan_matches_oracle(T, oracle, dim, n, nq):
+    O = oracle
+    oidx = OracleIndex(O, dim, 4, unit_gaussian(n, dim, seed=41))
+    q = unit_gaussian(nq, dim, seed=42)
+    ix = to_native(T, oidx)
+    rng = np.random.default_rng(6)
+    for m in (None, rng.random(n) < 0.5, rng.random(n) < 0.003, (np.arange(n) >= 9_000) & (np.arange(n) < 11_000)):
+        words = None if m is None else T.pack_mask(m)[0]
+        for k in (1, 10, 100):
+            s, i = ix.search(q, k, mask_words=words)
+            os_, oi = oidx.search(q, k, mask_words=words)
+            assert np.array_equal(i, oi), k
+            assert bits_equal(s, os_), k
+            ix.set_path(2)
+            s2, i2 = ix.search(q, k, mask_words=words)
+            ix.set_path(0)
+            assert np.array_equal(i2, i) and bits_equal(s2, s)
     ix.close()

@@ -218,7 +218,7 @@ class NativeIndex:
         return ms.value, n.value
 
     def set_path(self, force_full_lists):
-        check(lib().tv_debug_set_path(self.h, int(bool(force_full_lists))))
+        check(lib().tv_debug_set_path(self.h, int(force_full_lists)))
 
     def overflow_redos(self):
         c = C.c_size_t(0)

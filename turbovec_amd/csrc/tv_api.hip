@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <cstdlib>
 #include <new>
 #include <string>
 #include <vector>
@@ -355,6 +356,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
         Arena ar;
         ar.base = static_cast<uint8_t *>(ix->ws);
         Prepared pq;
+        size_t n_timed = 0;
         rc = prepare_queries(ix, ar, d_queries + q0 * g.dim, cq, pq);
         if (rc != TV_OK) return rc;
         int *d_tau = ar.take<int>(n_tiles * tv::kQTile);
@@ -364,39 +366,52 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
         TV_HIP(tv::launch_fill_i32(d_tau, int(0x807fffffu) /* order key of -inf */, n_tiles * tv::kQTile, ix->stream));
         TV_HIP(tv::launch_fill_i32(reinterpret_cast<int *>(d_over), 0, cq_pad, ix->stream));
 
+        const int nt_batched = (mode_p && cq > size_t(tv::kQTile) && !ix->no_batched) ? tv::batched_tiles(g.nch) : 0;
+        const int bgrid = tv::batched_grid_blocks(ix->device, g.nch);
         for (size_t lv = 0; lv < steps.size(); ++lv) {
             const bool last = lv + 1 == steps.size();
             const size_t level_blocks = (n_blocks + steps[lv] - 1) / steps[lv];
             // level 1 appends every slot it reads: two blocks per workgroup fill a segment exactly
             const int lgrid = int(std::min<size_t>(size_t(grid), std::max<size_t>(1, (level_blocks + 1) / 2)));
-            for (size_t t = 0; t < n_tiles; ++t) {
+            const bool batched = last && nt_batched > 0;
+            const size_t tiles_per_launch = batched ? size_t(nt_batched) : 1;
+            int n_seg = lgrid;
+            size_t launch_no = 0;
+            for (size_t t = 0; t < n_tiles; t += tiles_per_launch, ++launch_no) {
                 tv::ScanArgs a;
                 fill_scan_args(ix, a);
                 a.mask = d_mask;
                 a.tables = pq.d_tables + t * (mode_p ? pq.table_bytes_per_tile : tile_q * size_t(g.nch) * 1024);
                 a.qscale = pq.d_qscale + t * tile_q;
                 a.qbias = pq.d_qbias + t * tile_q;
-                a.nq_tile = int(std::min<size_t>(tile_q, cq - t * tile_q));
+                a.nq_tile = int(std::min<size_t>(tile_q * tiles_per_launch, cq - t * tile_q));
                 a.k = 1;
                 a.gtau = d_tau + t * tv::kQTile;
                 a.b_step = steps[lv];
                 a.cand = d_cand + t * tile_q * seg_stride * tv::kSegCap;
                 a.cand_cnt = d_cnt + t * tile_q * seg_stride;
                 a.seg_stride = uint32_t(seg_stride);
-                const bool timed = last && int(t) < kMaxTimedTiles;
-                if (timed) TV_HIP(hipEventRecord(g_events.start[t], ix->stream));
-                if (mode_p) TV_HIP(tv::launch_scan_p4(a, lgrid, tv::kModeAppend, ix->stream));
-                else TV_HIP(tv::launch_scan_lut(a, lgrid, tv::kModeAppend, ix->stream));
-                if (timed) TV_HIP(hipEventRecord(g_events.stop[t], ix->stream));
+                const bool timed = last && int(launch_no) < kMaxTimedTiles;
+                if (timed) TV_HIP(hipEventRecord(g_events.start[launch_no], ix->stream));
+                if (batched) {
+                    n_seg = int(std::min<size_t>(size_t(bgrid), seg_stride));
+                    TV_HIP(tv::launch_scan_p4_batched(a, n_seg, ix->stream));
+                } else if (mode_p) {
+                    TV_HIP(tv::launch_scan_p4(a, lgrid, tv::kModeAppend, ix->stream));
+                } else {
+                    TV_HIP(tv::launch_scan_lut(a, lgrid, tv::kModeAppend, ix->stream));
+                }
+                if (timed) TV_HIP(hipEventRecord(g_events.stop[launch_no], ix->stream));
             }
-            TV_HIP(tv::launch_final(d_cand, d_cnt, uint32_t(lgrid), uint32_t(seg_stride), int(k_eff), int(k_floor),
+            if (last) n_timed = std::min<size_t>(launch_no, size_t(kMaxTimedTiles));
+            TV_HIP(tv::launch_final(d_cand, d_cnt, uint32_t(n_seg), uint32_t(seg_stride), int(k_eff), int(k_floor),
                                     int(cq), d_out_scores + q0 * k_eff, d_out_idx + q0 * k_eff, d_over,
                                     last ? nullptr : d_tau, int(tile_q), ix->stream));
         }
         h_over.resize(cq);
         TV_HIP(hipMemcpyAsync(h_over.data(), d_over, cq * sizeof(uint32_t), hipMemcpyDeviceToHost, ix->stream));
         TV_HIP(hipStreamSynchronize(ix->stream));
-        for (size_t t = 0; t < n_tiles && int(t) < kMaxTimedTiles; ++t) {
+        for (size_t t = 0; t < n_timed; ++t) {
             float ms = 0.0f;
             TV_HIP(hipEventElapsedTime(&ms, g_events.start[t], g_events.stop[t]));
             ix->last_scan_ms += ms;
@@ -862,7 +877,8 @@ int tv_debug_stream_probe(tv_index *ix, const void *d_src, void *d_dst, size_t b
 
 int tv_debug_set_path(tv_index *ix, int force_full_lists) {
     if (!ix) return TV_ERR_BAD_ARGUMENT;
-    ix->force_robust = force_full_lists != 0;
+    ix->force_robust = (force_full_lists & 1) != 0;
+    ix->no_batched = (force_full_lists & 2) != 0;
     return TV_OK;
 }
 

@@ -95,6 +95,10 @@ int lut_tile_queries(int nch, int k);
 int lut_launch_ql(int nch, int k, int nq_tile);
 hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s);
 hipError_t launch_scan_lut(const ScanArgs &a, int grid, int mode, hipStream_t s);
+// Query tiles one batched permute-dot launch serves for this geometry (0: not available).
+int batched_tiles(int nch);
+int batched_grid_blocks(int device, int nch);
+hipError_t launch_scan_p4_batched(const ScanArgs &a, int grid, hipStream_t s);
 // out_tau == nullptr: write the k_eff best of the merged lists; else write only the
 // order key of the k_eff-th best (a floor at least k_eff scanned slots reach) per query.
 hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, const int *part_cnt, int total_threads,
@@ -146,5 +150,6 @@ struct tv_index {
     float last_scan_ms = 0.0f;
     int last_scan_launches = 0;
     int force_robust = 0;          // test hook: skip sample-then-filter
+    int no_batched = 0;            // test hook: one query tile per scan launch even for large batches
     size_t overflow_redos = 0;     // queries redone because their candidate buffer overflowed
 };

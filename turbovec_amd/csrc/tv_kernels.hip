@@ -8,8 +8,11 @@
 
 #include <cfloat>
 #include <climits>
+#include <cstdlib>
 
 namespace tv {
+
+static int batched_cfg();
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
@@ -390,6 +393,8 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
         const uint32_t b = j * step;
         v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         for (int c0 = 0; c0 < nch; c0 += U) {
+            // the next U chunks (of this block, or the head of the next one) are requested as one
+            // contiguous burst before the current U are consumed
             uint4 cur[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) cur[u] = buf[u];
@@ -492,6 +497,332 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
         __syncthreads();
         if (tid < a.nq_tile) a.cand_cnt[size_t(tid) * a.seg_stride + blockIdx.x] = scnt[tid];
     }
+}
+
+// ===========================================================================
+// Multi-tile scan, score mode P, append mode only: the weights of NT query
+// tiles stay resident in LDS for the whole launch (NT * dim bytes), every wave
+// decodes a chunk once and feeds NT tiles' MFMAs from it.  No barrier in the
+// main loop.  Used when NT * dim fits the 160 KiB of LDS.
+// ===========================================================================
+
+template <int NT, int U, int THREADS>
+__global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int nch = a.nch;
+    uint8_t *sW = smem;                                            // [NT][nch][2][64 lanes][16]
+    uint32_t *scnt = reinterpret_cast<uint32_t *>(smem + size_t(NT) * nch * 2048);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int qn = lane & 31, h = lane >> 5;
+    const int nt_active = (a.nq_tile + kQTile - 1) / kQTile;
+    {
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.tables);
+        uint4 *dst = reinterpret_cast<uint4 *>(sW);
+        const int live16 = nt_active * nch * 128;
+        for (int i = tid; i < NT * nch * 128; i += THREADS) dst[i] = i < live16 ? src[i] : make_uint4(0, 0, 0, 0);
+    }
+    for (int i = tid; i < NT * kQTile; i += THREADS) scnt[i] = 0u;
+    __syncthreads();
+
+    float qs[NT], qb[NT], tau[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int q = t * kQTile + qn;
+        const bool act = q < a.nq_tile;
+        qs[t] = act ? a.qscale[q] : 0.0f;
+        qb[t] = act ? a.qbias[q] : 0.0f;
+        tau[t] = act ? order_unkey(a.gtau[q]) : __int_as_float(0x7fc00000);  // NaN: nothing passes
+    }
+    const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
+
+    const uint32_t step = a.b_step;
+    const uint32_t nj = (a.n_blocks + step - 1) / step;
+    const uint32_t total_waves = gridDim.x * (THREADS / 64);
+    const uint32_t gw = wave * gridDim.x + blockIdx.x;             // consecutive blocks go to different workgroups
+    const uint4 *codes = reinterpret_cast<const uint4 *>(a.codes) + lane;
+    const uint4 *wlds = reinterpret_cast<const uint4 *>(sW) + lane;
+
+    auto live_from = [&](uint32_t j) -> uint32_t {
+        if (a.mask == nullptr) return j;
+        while (j < nj) {
+            const uint32_t b = j * step;
+            const uint64_t w = a.mask[b >> 1];
+            if (uint32_t(w >> ((b & 1) * 32)) != 0u) break;
+            j += total_waves;
+        }
+        return j;
+    };
+
+    uint32_t j = live_from(gw);
+    uint4 buf[U];
+    if (j < nj) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(j) * step * nch + u) * 64];
+    }
+    while (j < nj) {
+        const uint32_t nj_live = live_from(j + total_waves);
+        const uint32_t b = j * step;
+        v16i acc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (int c0 = 0; c0 < nch; c0 += U) {
+            // the next U chunks (of this block, or the head of the next one) are requested as one
+            // contiguous burst before the current U are consumed
+            uint4 cur[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) cur[u] = buf[u];
+            if (c0 + U < nch) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(b) * nch + c0 + U + u) * 64];
+            } else if (nj_live < nj) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(nj_live) * step * nch + u) * 64];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u;
+                const uint32_t x[4] = {cur[u].x, cur[u].y, cur[u].z, cur[u].w};
+                v4i alo, ahi;
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    alo[d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
+                    ahi[d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
+                }
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const uint4 wl = wlds[(size_t(t) * nch + c) * 128];
+                    const v4i blo = {int(wl.x), int(wl.y), int(wl.z), int(wl.w)};
+                    acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo, blo, acc[t], 0, 0, 0);
+                }
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const uint4 wh = wlds[(size_t(t) * nch + c) * 128 + 64];
+                    const v4i bhi = {int(wh.x), int(wh.y), int(wh.z), int(wh.w)};
+                    acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi, bhi, acc[t], 0, 0, 0);
+                }
+            }
+        }
+
+        const uint32_t slot0 = b * 32u;
+        uint32_t mw = 0xffffffffu;
+        if (a.mask != nullptr) mw = uint32_t(a.mask[b >> 1] >> ((b & 1) * 32));
+        float vs[16];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            const float4 f = *reinterpret_cast<const float4 *>(a.scales + slot0 + 8 * q4 + 4 * h);
+            vs[q4 * 4 + 0] = f.x; vs[q4 * 4 + 1] = f.y; vs[q4 * 4 + 2] = f.z; vs[q4 * 4 + 3] = f.w;
+        }
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float s = fmaf(float(acc[t][r]), qs[t], qb[t]) * vs[r];
+                if (s >= tau[t]) {
+                    const int i = 8 * (r >> 2) + 4 * h + (r & 3);
+                    const uint32_t slot = slot0 + i;
+                    if (slot < a.n && ((mw >> i) & 1u)) {
+                        const int q = t * kQTile + qn;
+                        const uint32_t pos = atomicAdd(&scnt[q], 1u);
+                        if (pos < kSegCap)
+                            a.cand[(size_t(q) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(s, slot);
+                    }
+                }
+            }
+        }
+        j = nj_live;
+    }
+    __syncthreads();
+    for (int q = tid; q < a.nq_tile; q += THREADS) a.cand_cnt[size_t(q) * a.seg_stride + blockIdx.x] = scnt[q];
+}
+
+// ===========================================================================
+// Batched scan, score mode P, append mode only: one pass serves NT query tiles
+// (NT*32 queries).  A workgroup walks groups of 4*MW blocks; each wave decodes
+// its MW blocks once per chunk and feeds NT tiles' MFMAs from the same decoded
+// operand, so the nibble decode -- the VALU cost that bounds the single-tile
+// kernel -- is amortised NT times.  The NT tiles' weights (NT * dim bytes) do
+// not fit LDS whole, so they stream through it in slices of KC chunks, double
+// buffered, shared by the four waves and re-read from L2 once per block group.
+// ===========================================================================
+
+template <int NT, int MW, int KC, int OCC>
+__global__ __launch_bounds__(kScanThreads, OCC) void k_scan_p4_batched(ScanArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int kSliceBytes = NT * KC * 2048;           // one slice of all tiles
+    constexpr int kStage = kSliceBytes / (kScanThreads * 16);  // uint4 per thread per slice
+    static_assert(kSliceBytes % (kScanThreads * 16) == 0, "slice must split evenly over the workgroup");
+    uint8_t *sB = smem;                                   // [2][NT][KC][2][1024]
+    uint32_t *scnt = reinterpret_cast<uint32_t *>(smem + 2 * kSliceBytes);  // [NT*32]
+    const int nch = a.nch;
+    const int nslices = nch / KC;                         // host guarantees nch % KC == 0
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int qn = lane & 31, h = lane >> 5;
+    const int nt_active = (a.nq_tile + kQTile - 1) / kQTile;
+    const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
+
+    for (int i = tid; i < NT * kQTile; i += kScanThreads) scnt[i] = 0u;
+
+    float qs[NT], qb[NT], tau[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int q = t * kQTile + qn;
+        const bool act = q < a.nq_tile;
+        qs[t] = act ? a.qscale[q] : 0.0f;
+        qb[t] = act ? a.qbias[q] : 0.0f;
+        tau[t] = act ? order_unkey(a.gtau[q]) : __int_as_float(0x7fc00000);  // NaN: nothing passes
+    }
+
+    const uint32_t step = a.b_step;
+    const uint32_t nj = (a.n_blocks + step - 1) / step;   // logical blocks
+    constexpr uint32_t kGroup = 4 * MW;                   // logical blocks per workgroup iteration
+    const uint32_t ngroups = (nj + kGroup - 1) / kGroup;
+
+    // staging of weight slices: thread copies kStage uint4 per slice; slice s of tile t lives at
+    // tables + t*nch*2048 + s*KC*2048 (KC*2048 contiguous bytes)
+    uint4 stage[kStage];
+    auto load_slice = [&](int sl) {
+#pragma unroll
+        for (int e = 0; e < kStage; ++e) {
+            const int idx = e * kScanThreads + tid;               // uint4 index within the slice
+            const int t = idx / (KC * 128), r = idx % (KC * 128);
+            if (t < nt_active)
+                stage[e] = reinterpret_cast<const uint4 *>(a.tables + (size_t(t) * nch + size_t(sl) * KC) * 2048)[r];
+            else
+                stage[e] = make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto store_slice = [&](int buf) {
+        uint4 *dst = reinterpret_cast<uint4 *>(sB + buf * kSliceBytes);
+#pragma unroll
+        for (int e = 0; e < kStage; ++e) dst[e * kScanThreads + tid] = stage[e];
+    };
+
+    const uint4 *codes = reinterpret_cast<const uint4 *>(a.codes) + lane;
+    uint32_t g = blockIdx.x;
+    if (g >= ngroups) {                                   // whole workgroup leaves together, with empty segments
+        for (int q = tid; q < a.nq_tile; q += kScanThreads) a.cand_cnt[size_t(q) * a.seg_stride + blockIdx.x] = 0u;
+        return;
+    }
+    load_slice(0);
+    store_slice(0);
+    __syncthreads();
+    int ring = 0;                                         // buffer holding the slice about to be consumed
+
+    for (; g < ngroups; g += gridDim.x) {
+        // this wave's MW logical blocks
+        uint32_t jb[MW];
+        bool live[MW];
+        uint32_t mw[MW];
+#pragma unroll
+        for (int m = 0; m < MW; ++m) {
+            jb[m] = g * kGroup + wave * MW + m;
+            live[m] = jb[m] < nj;
+            mw[m] = 0xffffffffu;
+            if (live[m] && a.mask != nullptr) {
+                const uint32_t b = jb[m] * step;
+                mw[m] = uint32_t(a.mask[b >> 1] >> ((b & 1) * 32));
+                live[m] = mw[m] != 0u;                    // block skip (search.rs:3015-3029)
+            }
+        }
+        v16i acc[MW][NT];
+#pragma unroll
+        for (int m = 0; m < MW; ++m)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[m][t] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+        uint4 abuf[MW][KC];                               // codes of the slice being computed
+#pragma unroll
+        for (int m = 0; m < MW; ++m)
+#pragma unroll
+            for (int c = 0; c < KC; ++c)
+                abuf[m][c] = live[m] ? codes[(size_t(jb[m]) * step * nch + c) * 64] : make_uint4(0, 0, 0, 0);
+
+        for (int sl = 0; sl < nslices; ++sl) {
+            const bool more = sl + 1 < nslices || g + gridDim.x < ngroups;
+            const int next_sl = sl + 1 < nslices ? sl + 1 : 0;
+            if (more) load_slice(next_sl);
+            uint4 acur[MW][KC];
+#pragma unroll
+            for (int m = 0; m < MW; ++m)
+#pragma unroll
+                for (int c = 0; c < KC; ++c) acur[m][c] = abuf[m][c];
+            if (sl + 1 < nslices) {
+#pragma unroll
+                for (int m = 0; m < MW; ++m)
+#pragma unroll
+                    for (int c = 0; c < KC; ++c)
+                        abuf[m][c] = live[m] ? codes[(size_t(jb[m]) * step * nch + (sl + 1) * KC + c) * 64]
+                                             : make_uint4(0, 0, 0, 0);
+            }
+            const uint4 *bl = reinterpret_cast<const uint4 *>(sB + ring * kSliceBytes) + lane;
+#pragma unroll
+            for (int c = 0; c < KC; ++c) {
+                v4i alo[MW], ahi[MW];
+#pragma unroll
+                for (int m = 0; m < MW; ++m) {
+                    const uint32_t x[4] = {acur[m][c].x, acur[m][c].y, acur[m][c].z, acur[m][c].w};
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        alo[m][d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
+                        ahi[m][d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
+                    }
+                }
+                // all low-nibble products first, then all high-nibble ones: the two MFMAs that
+                // chain on one accumulator end up NT*MW instructions apart instead of back to back
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const uint4 wl = bl[((t * KC + c) * 2) * 64];
+                    const v4i blo = {int(wl.x), int(wl.y), int(wl.z), int(wl.w)};
+#pragma unroll
+                    for (int m = 0; m < MW; ++m)
+                        acc[m][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo[m], blo, acc[m][t], 0, 0, 0);
+                }
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const uint4 wh = bl[((t * KC + c) * 2 + 1) * 64];
+                    const v4i bhi = {int(wh.x), int(wh.y), int(wh.z), int(wh.w)};
+#pragma unroll
+                    for (int m = 0; m < MW; ++m)
+                        acc[m][t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi[m], bhi, acc[m][t], 0, 0, 0);
+                }
+            }
+            if (more) store_slice(ring ^ 1);
+            __syncthreads();
+            ring ^= 1;
+        }
+
+        // ---- epilogue ----
+#pragma unroll
+        for (int m = 0; m < MW; ++m) {
+            if (!live[m]) continue;
+            const uint32_t slot0 = jb[m] * step * 32u;
+            float vs[16];
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const float4 f = *reinterpret_cast<const float4 *>(a.scales + slot0 + 8 * q4 + 4 * h);
+                vs[q4 * 4 + 0] = f.x; vs[q4 * 4 + 1] = f.y; vs[q4 * 4 + 2] = f.z; vs[q4 * 4 + 3] = f.w;
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float s = fmaf(float(acc[m][t][r]), qs[t], qb[t]) * vs[r];
+                    if (s >= tau[t]) {
+                        const int i = 8 * (r >> 2) + 4 * h + (r & 3);
+                        const uint32_t slot = slot0 + i;
+                        if (slot < a.n && ((mw[m] >> i) & 1u)) {
+                            const int q = t * kQTile + qn;
+                            const uint32_t pos = atomicAdd(&scnt[q], 1u);
+                            if (pos < kSegCap)
+                                a.cand[(size_t(q) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(s, slot);
+                        }
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (int q = tid; q < a.nq_tile; q += kScanThreads) a.cand_cnt[size_t(q) * a.seg_stride + blockIdx.x] = scnt[q];
 }
 
 // ===========================================================================
@@ -822,12 +1153,107 @@ hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s) 
         else if (mode == kModeAppend) { if (w_lds) TV_LAUNCH_P4(U, kModeAppend, true); else TV_LAUNCH_P4(U, kModeAppend, false); } \
         else { if (w_lds) TV_LAUNCH_P4(U, kModeLists, true); else TV_LAUNCH_P4(U, kModeLists, false); } \
     } while (0)
-    if (a.nch % 4 == 0) TV_PICK_P4(4);
+    if (a.nch % 8 == 0 && batched_cfg() >= 100) TV_PICK_P4(8);
+    else if (a.nch % 4 == 0) TV_PICK_P4(4);
     else if (a.nch % 2 == 0) TV_PICK_P4(2);
     else TV_PICK_P4(1);
 #undef TV_PICK_P4
 #undef TV_LAUNCH_P4
     return hipGetLastError();
+}
+
+// Batched append-mode launch for up to NT*32 queries (a.nq_tile counts queries, a.tables holds
+// ceil(nq/32) consecutive tiles).  Returns hipErrorInvalidValue when the geometry does not fit.
+static int batched_cfg() {
+    static int cfg = -1;
+    if (cfg < 0) {
+        const char *e = getenv("TV_BATCH_CFG");
+        cfg = e ? atoi(e) : 5;
+    }
+    return cfg;
+}
+
+// Query tiles whose weights fit LDS together (multi-tile kernel), capped at 4.
+static int resident_tiles(int nch) {
+    const size_t per_tile = size_t(nch) * 2048;
+    int nt = int((kLdsBudget - 1024) / per_tile);
+    return nt > 4 ? 4 : nt;
+}
+
+int batched_tiles(int nch) {
+    const int cfg = batched_cfg() % 100;
+    if (cfg < 10) {
+        const int nt = resident_tiles(nch);
+        if (nt >= 2) return nt;
+    }
+    const int kc = (cfg % 10 == 0) ? 4 : 2;
+    if (nch % kc != 0) return 0;
+    return (cfg % 10 == 2 || cfg % 10 == 3) ? 2 : 4;
+}
+
+int batched_grid_blocks(int device, int nch) {
+    hipDeviceProp_t prop;
+    int cus = 256;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0)
+        cus = prop.multiProcessorCount;
+    if (batched_cfg() % 100 < 10 && resident_tiles(nch) >= 2) {
+        const size_t lds = size_t(resident_tiles(nch)) * nch * 2048 + 1024;
+        int per_cu = int(kLdsBudget / lds);
+        return cus * (per_cu < 1 ? 1 : (per_cu > 2 ? 2 : per_cu));
+    }
+    return cus * (batched_cfg() % 100 % 10 == 0 ? 1 : 2);
+}
+
+template <int NT, int U, int THREADS>
+static hipError_t launch_multi_thr(const ScanArgs &a, int grid, hipStream_t s) {
+    const size_t lds = size_t(NT) * a.nch * 2048 + NT * kQTile * sizeof(uint32_t);
+    hipError_t e = allow_lds(k_scan_p4_multi<NT, U, THREADS>, lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((k_scan_p4_multi<NT, U, THREADS>), dim3(grid), dim3(THREADS), lds, s, a);
+    return hipGetLastError();
+}
+
+template <int NT, int U>
+static hipError_t launch_multi_cfg(const ScanArgs &a, int grid, hipStream_t s) {
+    const int cfg = batched_cfg() % 100;
+    if (cfg == 5) return launch_multi_thr<NT, U, 768>(a, grid, s);
+    if (cfg == 6) return launch_multi_thr<NT, U, 1024>(a, grid, s);
+    return launch_multi_thr<NT, U, 512>(a, grid, s);
+}
+
+template <int NT>
+static hipError_t launch_multi(const ScanArgs &a, int grid, hipStream_t s) {
+    if (a.nch % 8 == 0 && batched_cfg() >= 100) return launch_multi_cfg<NT, 8>(a, grid, s);
+    if (a.nch % 4 == 0) return launch_multi_cfg<NT, 4>(a, grid, s);
+    if (a.nch % 2 == 0) return launch_multi_cfg<NT, 2>(a, grid, s);
+    return launch_multi_cfg<NT, 1>(a, grid, s);
+}
+
+template <int NT, int MW, int KC, int OCC>
+static hipError_t launch_batched_cfg(const ScanArgs &a, int grid, hipStream_t s) {
+    if (a.nch % KC != 0 || a.nq_tile > NT * kQTile) return hipErrorInvalidValue;
+    const size_t lds = size_t(2) * NT * KC * 2048 + NT * kQTile * sizeof(uint32_t);
+    hipError_t e = allow_lds(k_scan_p4_batched<NT, MW, KC, OCC>, lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((k_scan_p4_batched<NT, MW, KC, OCC>), dim3(grid), dim3(kScanThreads), lds, s, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_scan_p4_batched(const ScanArgs &a, int grid, hipStream_t s) {
+    if (batched_cfg() % 100 < 10) {
+        switch (resident_tiles(a.nch)) {
+            case 4: return launch_multi<4>(a, grid, s);
+            case 3: return launch_multi<3>(a, grid, s);
+            case 2: return launch_multi<2>(a, grid, s);
+            default: break;
+        }
+    }
+    switch (batched_cfg() % 100 % 10) {
+        case 1: return launch_batched_cfg<4, 2, 2, 2>(a, grid, s);
+        case 2: return launch_batched_cfg<2, 2, 2, 2>(a, grid, s);
+        case 3: return launch_batched_cfg<2, 4, 2, 2>(a, grid, s);
+        default: return launch_batched_cfg<4, 2, 4, 1>(a, grid, s);
+    }
 }
 
 hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, const int *part_cnt, int total_threads,
