@@ -24,6 +24,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 
+# HBM bytes one launch of the dominant kernel moves (reads + writes), from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this same command, each scaled by the copy-probe factor (see profiles/).
+MEASURED_TRAFFIC = {}
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -34,6 +39,9 @@ def parse():
     ap.add_argument("--bits", type=int, default=4)
     ap.add_argument("--k", type=int, default=10)
     ap.add_argument("--batch", type=int, default=1024)
+    ap.add_argument("--score-mode", choices=["auto", "lut"], default="auto",
+                    help="auto = what the reference runs on a VNNI/dotprod host (int8 permute-dot at 4-bit); "
+                         "lut = the classic u8-LUT kernel's floats")
     ap.add_argument("--cpu-sample", type=int, default=2_000_000, help="vectors in the CPU-baseline sample (0 = skip)")
     ap.add_argument("--cpu-threads", type=int, default=16)
     ap.add_argument("--copy-probe", action="store_true",
@@ -102,6 +110,9 @@ def main():
     gen = torch.Generator(device=dev)
     gen.manual_seed(0)
     ix = T.NativeIndex(dim, bits)
+    if args.score_mode == "lut":
+        ix.set_score_mode(T.SCORE_L_CLASSIC)
+    mode_p = bits == 4 and args.score_mode == "auto"
     seq = torch.randint(0, 256, (n_blocks * G * 32,), dtype=torch.uint8, device=dev, generator=gen)
     scales = (torch.rand(n, device=dev, generator=gen) * 0.2 + 0.9).float()
     torch.cuda.synchronize()
@@ -143,13 +154,22 @@ def main():
     b1_steps = max(args.steps, 15)
     b1_launch_s = scan1_ms * 1e-3 / max(launches1, 1)
 
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "scan_traffic.json")
-    if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get(f"{n}x{dim}x{bits}")
-        except Exception:
-            traffic = None
+    # End-to-end rate when the boundary hands over host buffers (queries up, results down over PCIe).
+    import numpy as np
+    q_host = make_queries(args.batch).cpu().numpy()
+    ix.search(q_host, k)
+    t0 = time.perf_counter()
+    for _ in range(3):
+        ix.search(q_host, k)
+    host_qps = 3 * args.batch / (time.perf_counter() - t0)
+
+    q_per_launch = args.batch * args.steps / max(launches, 1)
+    if mode_p:
+        kernel = "k_scan_p4_multi" if q_per_launch > 32 else "k_scan_p4"
+    else:
+        kernel = "k_scan_lut"
+    traffic = MEASURED_TRAFFIC.get((kernel, n, dim, bits))
+    int8_ops = 2.0 * q_per_launch * n * dim        # multiply-adds x2 of one launch, permute-dot mode
 
     out = {
         "metric": "queries/sec, 10Mx1536 4-bit, k=10 (batch 1024; batch 1 beside it)",
@@ -162,22 +182,28 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8",
+        "dtype": "int8" if mode_p else "u8",
         "data": "synthetic",
         "config": {"workload": f"TurboQuantIndex {n}x{dim} {bits}-bit, k={k}, no filter, batch {args.batch}",
-                   "score_mode": "permute-dot (int8 weights x int8 codebook levels, i32 accumulate)" if bits == 4
-                   else "u8 LUT, u32 accumulate", "n": n, "dim": dim, "bits": bits, "k": k, "batch": args.batch},
+                   "score_mode": "permute-dot (int8 weights x int8 codebook levels, i32 accumulate)" if mode_p
+                   else "u8 LUT, integer accumulate", "n": n, "dim": dim, "bits": bits, "k": k, "batch": args.batch},
         "batch1": {"queries_per_s": b1_steps / dt1, "ms_per_query": dt1 / b1_steps * 1e3,
                    "scan_kernel_ms": b1_launch_s * 1e3, "achieved_GBps": alg_bytes / b1_launch_s / 1e9,
                    "frac_of_hbm_peak": alg_bytes / b1_launch_s / 1e9 / 8000.0,
                    "frac_of_achievable": alg_bytes / b1_launch_s / 1e9 / read_probe},
+        "host_buffers": {"queries_per_s": host_qps,
+                         "note": "same batch through tv_search with host query/result buffers (PCIe both ways)"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s",
                      "frac": achieved / 8000.0, "traffic": traffic,
-                     "kernel": "k_scan_p4" if bits == 4 else "k_scan_lut",
+                     "kernel": kernel,
                      "achievable_read_GBps": read_probe, "frac_of_achievable": achieved / read_probe,
                      "algorithmic_bytes_per_launch": alg_bytes, "launches_timed": launches,
-                     "mean_launch_ms": launch_s * 1e3, "queries_per_launch": 32 if bits == 4 else None},
+                     "mean_launch_ms": launch_s * 1e3, "queries_per_launch": q_per_launch},
     }
+    if mode_p:
+        out["mfma"] = {"achieved": int8_ops / launch_s / 1e12, "peak": 5000.0, "unit": "TOP/s",
+                       "frac": int8_ops / launch_s / 1e12 / 5000.0,
+                       "note": "int8 multiply-adds x2 of the queries one launch scores, over the same launch time"}
     if args.cpu_sample > 0:
         out["cpu_baseline"] = cpu_baseline(args)
     print(json.dumps(out))

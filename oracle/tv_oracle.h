@@ -21,16 +21,23 @@
  *   tvo_fit_calibration,
  *   tvo_encode, tvo_norm     pinned: calibration/codes/scales hashes, 8 cells.
  *   tvo_repack_seq et al.    pinned: closed-form byte maps (src/pack.rs:964-1008).
- *   tvo_build_permute_dot    pinned: slot map + zero identity (src/search.rs:4596)
- *                            and end-to-end by the parity fixture.
- *   tvo_build_lut            PARITY UNPINNED beyond invariants (entries <= 127,
- *                            power-of-two scaling invariance, zero query); the
- *                            reference holds no golden LUT bytes.
- *   tvo_search  mode P       pinned: 600 float scores + ids of
- *                            benchmarks/hillclimb/data/parity_base_x86.json.
- *   tvo_search  modes L_*    PARITY UNPINNED end-to-end (no reference-held
- *                            vectors for 2-bit or classic 4-bit); integer sums are
- *                            checked by brute force against decoded codes.
+ *   tvo_build_lut            pinned end to end through the parity fixture below (any
+ *                            wrong entry, scale or bias moves one of its 600 floats);
+ *                            2-/3-bit tables: PARITY UNPINNED beyond invariants
+ *                            (entries <= 127, power-of-two scaling, zero query).
+ *   tvo_search  L_CLASSIC    pinned at 4-bit: the 3 x 200 float scores and ids of
+ *                            benchmarks/hillclimb/data/parity_base_{x86,arm}.json are
+ *                            reproduced bit for bit (base, after the warm appends,
+ *                            after 500 swap-removes).
+ *   tvo_build_permute_dot    slot map and zero identity pinned (src/search.rs:4596);
+ *   tvo_search  mode P       end-to-end floats PARITY UNPINNED: the reference holds no
+ *                            vector produced by its int8 permute-dot kernel (the fixture
+ *                            above was written by the LUT kernel).  Integer dots are
+ *                            checked by brute force against decoded codes; ranking
+ *                            agrees with the fixture up to quantisation of the weights.
+ *   tvo_search  L_U32,       PARITY UNPINNED end to end; they share the pinned LUT and
+ *               L_SCALAR     integer sums with L_CLASSIC, the epilogue follows
+ *                            search.rs:1174-1177 / 3077-3147 line by line.
  */
 #ifndef TV_ORACLE_H
 #define TV_ORACLE_H

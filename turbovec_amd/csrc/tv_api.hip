@@ -373,7 +373,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             const size_t level_blocks = (n_blocks + steps[lv] - 1) / steps[lv];
             // level 1 appends every slot it reads: two blocks per workgroup fill a segment exactly
             const int lgrid = int(std::min<size_t>(size_t(grid), std::max<size_t>(1, (level_blocks + 1) / 2)));
-            const bool batched = last && nt_batched > 0;
+            const bool batched = nt_batched > 0;
             const size_t tiles_per_launch = batched ? size_t(nt_batched) : 1;
             int n_seg = lgrid;
             size_t launch_no = 0;

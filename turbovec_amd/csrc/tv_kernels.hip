@@ -314,6 +314,33 @@ __global__ __launch_bounds__(256) void k_build_lut(const float *__restrict__ qca
 // score = fma(f32(acc), scale, bias) * vec_scale (search.rs:1519-1524).
 // ===========================================================================
 
+// ---------------------------------------------------------------------------
+// Hand-placed code loads.  The vector-memory counter retires in order, and the
+// compiler's own wait placement is decided per merge point of the control flow,
+// which for a software-pipelined stream ends up waiting on the burst it has
+// just issued.  These loads are invisible to that pass: the kernel states how
+// many younger loads may stay in flight where it consumes a register
+// (wait_vm<N>).  Loads the compiler issues itself only make its own waits
+// stricter, never looser, because a count is an upper bound on what may remain.
+// ---------------------------------------------------------------------------
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <int OFF>
+__device__ __forceinline__ void load16_async(u32x4 &dst, const void *p) {
+    asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(dst) : "v"(p), "n"(OFF));
+}
+__device__ __forceinline__ void load4_async(float &dst, const void *p) {
+    asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(p));
+}
+template <int N>
+__device__ __forceinline__ void wait_vm(u32x4 &r) {
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(r) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_vm(float &r) {
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(r) : "n"(N));
+}
+
 // Four packed nibbles (one per byte, values 0..15) -> four int8 levels.
 // v_perm_b32 looks up 8 table bytes; selectors >= 13 give 0xff, so each half
 // of the 16-entry table is looked up with the other half's nibbles pushed out
@@ -522,6 +549,8 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
         for (int i = tid; i < NT * nch * 128; i += THREADS) dst[i] = i < live16 ? src[i] : make_uint4(0, 0, 0, 0);
     }
     for (int i = tid; i < NT * kQTile; i += THREADS) scnt[i] = 0u;
+    uint32_t *snext = scnt + NT * kQTile;   // next unclaimed block of this workgroup
+    if (tid == 0) *snext = 0u;
     __syncthreads();
 
     float qs[NT], qb[NT], tau[NT];
@@ -532,93 +561,70 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
         qs[t] = act ? a.qscale[q] : 0.0f;
         qb[t] = act ? a.qbias[q] : 0.0f;
         tau[t] = act ? order_unkey(a.gtau[q]) : __int_as_float(0x7fc00000);  // NaN: nothing passes
+        // Pass the three through a register move the compiler cannot see through: it then waits
+        // for these loads here, once, instead of before their first use inside the stream, where
+        // a full wait would also drain the code loads in flight.
+        asm volatile("v_mov_b32 %0, %0\n v_mov_b32 %1, %1\n v_mov_b32 %2, %2" : "+v"(qs[t]), "+v"(qb[t]), "+v"(tau[t]));
     }
     const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
 
     const uint32_t step = a.b_step;
     const uint32_t nj = (a.n_blocks + step - 1) / step;
-    const uint32_t total_waves = gridDim.x * (THREADS / 64);
-    const uint32_t gw = wave * gridDim.x + blockIdx.x;             // consecutive blocks go to different workgroups
     const uint4 *codes = reinterpret_cast<const uint4 *>(a.codes) + lane;
     const uint4 *wlds = reinterpret_cast<const uint4 *>(sW) + lane;
 
-    auto live_from = [&](uint32_t j) -> uint32_t {
-        if (a.mask == nullptr) return j;
-        while (j < nj) {
+    // Blocks are dealt round-robin to workgroups (logical block m * gridDim.x + blockIdx.x belongs
+    // to this one), so neighbouring rows -- clustered data, contiguous allowlists -- spread over
+    // all of them; inside a workgroup the waves claim blocks from a shared counter as they go,
+    // so all of them finish within one block of each other whatever the SIMD arbitration did.
+    // Returns the next block with at least one allowed slot (search.rs:3015-3029), or >= nj.
+    auto claim = [&]() -> uint32_t {
+        for (;;) {
+            uint32_t m = 0;
+            if (lane == 0) m = atomicAdd(snext, 1u);
+            m = uint32_t(__builtin_amdgcn_readfirstlane(int(m)));
+            const uint32_t j = m * gridDim.x + blockIdx.x;
+            if (j >= nj || a.mask == nullptr) return j;
             const uint32_t b = j * step;
-            const uint64_t w = a.mask[b >> 1];
-            if (uint32_t(w >> ((b & 1) * 32)) != 0u) break;
-            j += total_waves;
+            if (uint32_t(a.mask[b >> 1] >> ((b & 1) * 32)) != 0u) return j;
         }
-        return j;
     };
 
-    uint32_t j = live_from(gw);
-    uint4 buf[U];
-    if (j < nj) {
+    // The wave's work is one stream of U-chunk groups running through its blocks.  Two register
+    // sets take turns: while one group is decoded and multiplied, the next group's codes (of this
+    // block, or the head of the next live one) are in flight into the other set, requested as one
+    // contiguous burst.  Every group issues the same loads in the same order -- the row scale of
+    // its block, then the burst -- so the number of younger loads behind any register is fixed:
+    // before chunk u of the current set, 2U - u of them may still be outstanding.
+    v16i acc[NT];
 #pragma unroll
-        for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(j) * step * nch + u) * 64];
-    }
-    while (j < nj) {
-        const uint32_t nj_live = live_from(j + total_waves);
-        const uint32_t b = j * step;
-        v16i acc[NT];
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        for (int c0 = 0; c0 < nch; c0 += U) {
-            // the next U chunks (of this block, or the head of the next one) are requested as one
-            // contiguous burst before the current U are consumed
-            uint4 cur[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u) cur[u] = buf[u];
-            if (c0 + U < nch) {
-#pragma unroll
-                for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(b) * nch + c0 + U + u) * 64];
-            } else if (nj_live < nj) {
-#pragma unroll
-                for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(nj_live) * step * nch + u) * 64];
-            }
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int c = c0 + u;
-                const uint32_t x[4] = {cur[u].x, cur[u].y, cur[u].z, cur[u].w};
-                v4i alo, ahi;
-#pragma unroll
-                for (int d = 0; d < 4; ++d) {
-                    alo[d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
-                    ahi[d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
-                }
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const uint4 wl = wlds[(size_t(t) * nch + c) * 128];
-                    const v4i blo = {int(wl.x), int(wl.y), int(wl.z), int(wl.w)};
-                    acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo, blo, acc[t], 0, 0, 0);
-                }
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const uint4 wh = wlds[(size_t(t) * nch + c) * 128 + 64];
-                    const v4i bhi = {int(wh.x), int(wh.y), int(wh.z), int(wh.w)};
-                    acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi, bhi, acc[t], 0, 0, 0);
-                }
-            }
-        }
+    for (int t = 0; t < NT; ++t) acc[t] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    uint32_t j = claim();
+    int c0 = 0;
+    const uint8_t *code_bytes = reinterpret_cast<const uint8_t *>(codes);   // lane offset included
 
+    auto issue = [&](u32x4 (&dst)[U], float &sc, uint32_t jb_phys, int c) {
+        load4_async(sc, a.scales + jb_phys * 32u + qn);
+        const uint8_t *p = code_bytes + (size_t(jb_phys) * nch + c) * 1024;
+        load16_async<0>(dst[0], p);
+        if (U > 1) load16_async<1024>(dst[U > 1 ? 1 : 0], p);
+        if (U > 2) load16_async<2048>(dst[U > 2 ? 2 : 0], p);
+        if (U > 3) load16_async<3072>(dst[U > 3 ? 3 : 0], p);
+        static_assert(U <= 4, "immediate offsets cover four chunks");
+    };
+
+    auto finish_block = [&](uint32_t b, float my_scale) {
         const uint32_t slot0 = b * 32u;
         uint32_t mw = 0xffffffffu;
         if (a.mask != nullptr) mw = uint32_t(a.mask[b >> 1] >> ((b & 1) * 32));
-        float vs[16];
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-            const float4 f = *reinterpret_cast<const float4 *>(a.scales + slot0 + 8 * q4 + 4 * h);
-            vs[q4 * 4 + 0] = f.x; vs[q4 * 4 + 1] = f.y; vs[q4 * 4 + 2] = f.z; vs[q4 * 4 + 3] = f.w;
-        }
+        for (int r = 0; r < 16; ++r) {
+            const int i = 8 * (r >> 2) + 4 * h + (r & 3);
+            const float vsr = __shfl(my_scale, i);
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float s = fmaf(float(acc[t][r]), qs[t], qb[t]) * vs[r];
+            for (int t = 0; t < NT; ++t) {
+                const float s = fmaf(float(acc[t][r]), qs[t], qb[t]) * vsr;
                 if (s >= tau[t]) {
-                    const int i = 8 * (r >> 2) + 4 * h + (r & 3);
                     const uint32_t slot = slot0 + i;
                     if (slot < a.n && ((mw >> i) & 1u)) {
                         const int q = t * kQTile + qn;
@@ -629,7 +635,62 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
                 }
             }
         }
-        j = nj_live;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    };
+
+    // One group: request the following group into `nxt`, consume `cur`.  Returns false after the
+    // wave's last group (whose request re-reads the current group: a valid address, never used).
+    auto phase = [&](u32x4 (&cur)[U], float &cur_sc, u32x4 (&nxt)[U], float &nxt_sc) -> bool {
+        const uint32_t b = j * step;
+        const bool block_ends = c0 + U >= nch;
+        uint32_t pj = j;
+        int pc = c0 + U;
+        if (block_ends) { pj = claim(); pc = 0; }
+        const bool more = pj < nj;
+        issue(nxt, nxt_sc, (more ? pj : j) * step, more ? pc : c0);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u;
+            if (u == 0) wait_vm<2 * U - 0>(cur[0]);
+            if (u == 1) wait_vm<2 * U - 1>(cur[U > 1 ? 1 : 0]);
+            if (u == 2) wait_vm<2 * U - 2>(cur[U > 2 ? 2 : 0]);
+            if (u == 3) wait_vm<2 * U - 3>(cur[U > 3 ? 3 : 0]);
+            const uint32_t x[4] = {cur[u].x, cur[u].y, cur[u].z, cur[u].w};
+            v4i alo, ahi;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                alo[d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
+                ahi[d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const uint4 wl = wlds[(size_t(t) * nch + c) * 128];
+                const v4i blo = {int(wl.x), int(wl.y), int(wl.z), int(wl.w)};
+                acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo, blo, acc[t], 0, 0, 0);
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const uint4 wh = wlds[(size_t(t) * nch + c) * 128 + 64];
+                const v4i bhi = {int(wh.x), int(wh.y), int(wh.z), int(wh.w)};
+                acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi, bhi, acc[t], 0, 0, 0);
+            }
+        }
+        if (block_ends) {
+            wait_vm<U + 1>(cur_sc);   // this group's own scale: only the request issued above is younger
+            finish_block(b, cur_sc);
+        }
+        j = pj;
+        c0 = pc;
+        return more;
+    };
+
+    if (j < nj) {
+        u32x4 bufA[U], bufB[U];
+        float scA, scB;
+        issue(bufA, scA, j * step, 0);
+        while (phase(bufA, scA, bufB, scB) && phase(bufB, scB, bufA, scA)) {}
+        asm volatile("s_waitcnt vmcnt(0)");
     }
     __syncthreads();
     for (int q = tid; q < a.nq_tile; q += THREADS) a.cand_cnt[size_t(q) * a.seg_stride + blockIdx.x] = scnt[q];
@@ -1206,7 +1267,7 @@ int batched_grid_blocks(int device, int nch) {
 
 template <int NT, int U, int THREADS>
 static hipError_t launch_multi_thr(const ScanArgs &a, int grid, hipStream_t s) {
-    const size_t lds = size_t(NT) * a.nch * 2048 + NT * kQTile * sizeof(uint32_t);
+    const size_t lds = size_t(NT) * a.nch * 2048 + (NT * kQTile + 1) * sizeof(uint32_t);
     hipError_t e = allow_lds(k_scan_p4_multi<NT, U, THREADS>, lds);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((k_scan_p4_multi<NT, U, THREADS>), dim3(grid), dim3(THREADS), lds, s, a);
@@ -1223,7 +1284,6 @@ static hipError_t launch_multi_cfg(const ScanArgs &a, int grid, hipStream_t s) {
 
 template <int NT>
 static hipError_t launch_multi(const ScanArgs &a, int grid, hipStream_t s) {
-    if (a.nch % 8 == 0 && batched_cfg() >= 100) return launch_multi_cfg<NT, 8>(a, grid, s);
     if (a.nch % 4 == 0) return launch_multi_cfg<NT, 4>(a, grid, s);
     if (a.nch % 2 == 0) return launch_multi_cfg<NT, 2>(a, grid, s);
     return launch_multi_cfg<NT, 1>(a, grid, s);
