@@ -539,7 +539,7 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
     const int nch = a.nch;
     uint8_t *sW = smem;                                            // [NT][nch][2][64 lanes][16]
     uint32_t *scnt = reinterpret_cast<uint32_t *>(smem + size_t(NT) * nch * 2048);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
     const int qn = lane & 31, h = lane >> 5;
     const int nt_active = (a.nq_tile + kQTile - 1) / kQTile;
     {
@@ -617,21 +617,22 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
         const uint32_t slot0 = b * 32u;
         uint32_t mw = 0xffffffffu;
         if (a.mask != nullptr) mw = uint32_t(a.mask[b >> 1] >> ((b & 1) * 32));
+        // Rows past the end of the index or outside the allowlist get a NaN scale: their scores
+        // then fail the floor compare by themselves, and the per-score path has no other test.
+        if (slot0 + 32u > a.n) mw &= (a.n > slot0) ? (0xffffffffu >> (slot0 + 32u - a.n)) : 0u;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int i = 8 * (r >> 2) + 4 * h + (r & 3);
-            const float vsr = __shfl(my_scale, i);
+            float vsr = __shfl(my_scale, i);
+            if (!((mw >> i) & 1u)) vsr = __int_as_float(0x7fc00000);
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 const float s = fmaf(float(acc[t][r]), qs[t], qb[t]) * vsr;
                 if (s >= tau[t]) {
-                    const uint32_t slot = slot0 + i;
-                    if (slot < a.n && ((mw >> i) & 1u)) {
-                        const int q = t * kQTile + qn;
-                        const uint32_t pos = atomicAdd(&scnt[q], 1u);
-                        if (pos < kSegCap)
-                            a.cand[(size_t(q) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(s, slot);
-                    }
+                    const int q = t * kQTile + qn;
+                    const uint32_t pos = atomicAdd(&scnt[q], 1u);
+                    if (pos < kSegCap)
+                        a.cand[(size_t(q) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(s, slot0 + i);
                 }
             }
         }
