@@ -12,7 +12,6 @@
 
 namespace tv {
 
-static int batched_cfg();
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
@@ -1215,8 +1214,7 @@ hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s) 
         else if (mode == kModeAppend) { if (w_lds) TV_LAUNCH_P4(U, kModeAppend, true); else TV_LAUNCH_P4(U, kModeAppend, false); } \
         else { if (w_lds) TV_LAUNCH_P4(U, kModeLists, true); else TV_LAUNCH_P4(U, kModeLists, false); } \
     } while (0)
-    if (a.nch % 8 == 0 && batched_cfg() >= 100) TV_PICK_P4(8);
-    else if (a.nch % 4 == 0) TV_PICK_P4(4);
+    if (a.nch % 4 == 0) TV_PICK_P4(4);
     else if (a.nch % 2 == 0) TV_PICK_P4(2);
     else TV_PICK_P4(1);
 #undef TV_PICK_P4
@@ -1224,33 +1222,25 @@ hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s) 
     return hipGetLastError();
 }
 
-// Batched append-mode launch for up to NT*32 queries (a.nq_tile counts queries, a.tables holds
-// ceil(nq/32) consecutive tiles).  Returns hipErrorInvalidValue when the geometry does not fit.
-static int batched_cfg() {
-    static int cfg = -1;
-    if (cfg < 0) {
-        const char *e = getenv("TV_BATCH_CFG");
-        cfg = e ? atoi(e) : 5;
-    }
-    return cfg;
-}
+// Batched append-mode launches for up to batched_tiles()*32 queries (a.nq_tile counts queries,
+// a.tables holds ceil(nq/32) consecutive tiles).  Two kernels: when the weights of at least two
+// tiles fit LDS together they stay resident (k_scan_p4_multi); wider rows stream four tiles'
+// weights through LDS in slices (k_scan_p4_batched).
 
-// Query tiles whose weights fit LDS together (multi-tile kernel), capped at 4.
+// Query tiles whose weights fit LDS together, capped at 4.
 static int resident_tiles(int nch) {
     const size_t per_tile = size_t(nch) * 2048;
     int nt = int((kLdsBudget - 1024) / per_tile);
     return nt > 4 ? 4 : nt;
 }
 
+constexpr int kMultiThreads = 768;   // 3 waves per SIMD: measured best of 512 / 768 / 1024
+constexpr int kStreamTiles = 4, kStreamBlocksPerWave = 2, kStreamSliceChunks = 2, kStreamOccupancy = 2;
+
 int batched_tiles(int nch) {
-    const int cfg = batched_cfg() % 100;
-    if (cfg < 10) {
-        const int nt = resident_tiles(nch);
-        if (nt >= 2) return nt;
-    }
-    const int kc = (cfg % 10 == 0) ? 4 : 2;
-    if (nch % kc != 0) return 0;
-    return (cfg % 10 == 2 || cfg % 10 == 3) ? 2 : 4;
+    const int nt = resident_tiles(nch);
+    if (nt >= 2) return nt;
+    return nch % kStreamSliceChunks == 0 ? kStreamTiles : 0;
 }
 
 int batched_grid_blocks(int device, int nch) {
@@ -1258,63 +1248,44 @@ int batched_grid_blocks(int device, int nch) {
     int cus = 256;
     if (hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0)
         cus = prop.multiProcessorCount;
-    if (batched_cfg() % 100 < 10 && resident_tiles(nch) >= 2) {
+    if (resident_tiles(nch) >= 2) {
         const size_t lds = size_t(resident_tiles(nch)) * nch * 2048 + 1024;
-        int per_cu = int(kLdsBudget / lds);
+        const int per_cu = int(kLdsBudget / lds);
         return cus * (per_cu < 1 ? 1 : (per_cu > 2 ? 2 : per_cu));
     }
-    return cus * (batched_cfg() % 100 % 10 == 0 ? 1 : 2);
-}
-
-template <int NT, int U, int THREADS>
-static hipError_t launch_multi_thr(const ScanArgs &a, int grid, hipStream_t s) {
-    const size_t lds = size_t(NT) * a.nch * 2048 + (NT * kQTile + 1) * sizeof(uint32_t);
-    hipError_t e = allow_lds(k_scan_p4_multi<NT, U, THREADS>, lds);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((k_scan_p4_multi<NT, U, THREADS>), dim3(grid), dim3(THREADS), lds, s, a);
-    return hipGetLastError();
+    return cus * kStreamOccupancy;
 }
 
 template <int NT, int U>
-static hipError_t launch_multi_cfg(const ScanArgs &a, int grid, hipStream_t s) {
-    const int cfg = batched_cfg() % 100;
-    if (cfg == 5) return launch_multi_thr<NT, U, 768>(a, grid, s);
-    if (cfg == 6) return launch_multi_thr<NT, U, 1024>(a, grid, s);
-    return launch_multi_thr<NT, U, 512>(a, grid, s);
+static hipError_t launch_multi_u(const ScanArgs &a, int grid, hipStream_t s) {
+    const size_t lds = size_t(NT) * a.nch * 2048 + (NT * kQTile + 1) * sizeof(uint32_t);
+    hipError_t e = allow_lds(k_scan_p4_multi<NT, U, kMultiThreads>, lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((k_scan_p4_multi<NT, U, kMultiThreads>), dim3(grid), dim3(kMultiThreads), lds, s, a);
+    return hipGetLastError();
 }
 
 template <int NT>
 static hipError_t launch_multi(const ScanArgs &a, int grid, hipStream_t s) {
-    if (a.nch % 4 == 0) return launch_multi_cfg<NT, 4>(a, grid, s);
-    if (a.nch % 2 == 0) return launch_multi_cfg<NT, 2>(a, grid, s);
-    return launch_multi_cfg<NT, 1>(a, grid, s);
+    if (a.nch % 4 == 0) return launch_multi_u<NT, 4>(a, grid, s);
+    if (a.nch % 2 == 0) return launch_multi_u<NT, 2>(a, grid, s);
+    return launch_multi_u<NT, 1>(a, grid, s);
 }
 
-template <int NT, int MW, int KC, int OCC>
-static hipError_t launch_batched_cfg(const ScanArgs &a, int grid, hipStream_t s) {
+hipError_t launch_scan_p4_batched(const ScanArgs &a, int grid, hipStream_t s) {
+    switch (resident_tiles(a.nch)) {
+        case 4: return launch_multi<4>(a, grid, s);
+        case 3: return launch_multi<3>(a, grid, s);
+        case 2: return launch_multi<2>(a, grid, s);
+        default: break;
+    }
+    constexpr int NT = kStreamTiles, MW = kStreamBlocksPerWave, KC = kStreamSliceChunks, OCC = kStreamOccupancy;
     if (a.nch % KC != 0 || a.nq_tile > NT * kQTile) return hipErrorInvalidValue;
     const size_t lds = size_t(2) * NT * KC * 2048 + NT * kQTile * sizeof(uint32_t);
     hipError_t e = allow_lds(k_scan_p4_batched<NT, MW, KC, OCC>, lds);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((k_scan_p4_batched<NT, MW, KC, OCC>), dim3(grid), dim3(kScanThreads), lds, s, a);
     return hipGetLastError();
-}
-
-hipError_t launch_scan_p4_batched(const ScanArgs &a, int grid, hipStream_t s) {
-    if (batched_cfg() % 100 < 10) {
-        switch (resident_tiles(a.nch)) {
-            case 4: return launch_multi<4>(a, grid, s);
-            case 3: return launch_multi<3>(a, grid, s);
-            case 2: return launch_multi<2>(a, grid, s);
-            default: break;
-        }
-    }
-    switch (batched_cfg() % 100 % 10) {
-        case 1: return launch_batched_cfg<4, 2, 2, 2>(a, grid, s);
-        case 2: return launch_batched_cfg<2, 2, 2, 2>(a, grid, s);
-        case 3: return launch_batched_cfg<2, 4, 2, 2>(a, grid, s);
-        default: return launch_batched_cfg<4, 2, 4, 1>(a, grid, s);
-    }
 }
 
 hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, const int *part_cnt, int total_threads,
