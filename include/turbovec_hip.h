@@ -87,6 +87,16 @@ int tv_index_upload_seq_dev(tv_index *ix, const uint8_t *d_seq_codes, size_t n_v
  * per-vector form extract_codes_flat yields, pack.rs:306).  Replaces
  * append_lanes (pack.rs:211-233). */
 int tv_index_append_rows(tv_index *ix, const uint8_t *rows, const float *scales, size_t n_new);
+/* Encode n_new raw float rows (n_new*dim values) on the device and append them:
+ * normalise, rotate, quantise against the codebook (and the TQ+ pair when one is
+ * set), derive the per-vector scale, pack, append.  Codes and scales are
+ * bit-identical to the CPU encoder's.  Replaces the encode half of
+ * TurboQuantIndex::add (lib.rs:738-966 -> encode.rs:1418-1476, :560-664,
+ * :900-932).  Values must be finite with |x| < 1e16 (encode.rs:76-83):
+ * TV_ERR_INVALID_QUERY_VALUE otherwise, and nothing is added. */
+int tv_index_add(tv_index *ix, const float *vectors, size_t n_new);
+/* Same, rows already in device memory (not validated: the caller checked them). */
+int tv_index_add_dev(tv_index *ix, const float *d_vectors, size_t n_new);
 /* lib.rs:2864-3028: move the last vector into slot idx, zero the vacated lane. */
 int tv_index_swap_remove(tv_index *ix, size_t idx);
 /* Copy the index back in the sequential-blocked layout (codes_blocked_seq,

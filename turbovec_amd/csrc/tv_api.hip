@@ -637,6 +637,61 @@ int tv_index_append_rows(tv_index *ix, const uint8_t *rows, const float *scales,
     return TV_OK;
 }
 
+// lib.rs add -> encode.rs:1418-1476 on the device, then append_lanes (pack.rs:211-233).
+static int add_device_rows(tv_index *ix, const float *d_vectors, size_t n_new) {
+    const tv::Geometry &g = ix->geo;
+    const bool cal = !ix->tq_shift.empty();
+    const size_t slice = size_t(1) << 20;
+    for (size_t r0 = 0; r0 < n_new; r0 += slice) {
+        const size_t nr = std::min(slice, n_new - r0);
+        TV_HIP(tv::launch_encode(d_vectors + r0 * size_t(g.dim), nr, ix->n + r0, ix->d_signs, ix->d_perms,
+                                 cal ? ix->d_tq_shift : nullptr, cal ? ix->d_tq_scale : nullptr,
+                                 ix->cb.centroids.data(), ix->cb.boundaries.data(), g, ix->rot.block,
+                                 ix->rot.inv_sqrt_block, ix->d_codes, ix->d_scales, ix->stream));
+    }
+    TV_HIP(hipStreamSynchronize(ix->stream));
+    ix->n += n_new;
+    return TV_OK;
+}
+
+int tv_index_add_dev(tv_index *ix, const float *d_vectors, size_t n_new) {
+    if (!ix || (n_new && !d_vectors)) return TV_ERR_BAD_ARGUMENT;
+    if (n_new == 0) return TV_OK;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    if (ix->n + n_new >= (size_t(1) << 31)) return TV_ERR_BAD_ARGUMENT;
+    int rc = ensure_capacity(ix, ix->n + n_new);
+    if (rc != TV_OK) return rc;
+    return add_device_rows(ix, d_vectors, n_new);
+}
+
+int tv_index_add(tv_index *ix, const float *vectors, size_t n_new) {
+    if (!ix || (n_new && !vectors)) return TV_ERR_BAD_ARGUMENT;
+    if (n_new == 0) return TV_OK;
+    const size_t dim = size_t(ix->geo.dim);
+    size_t bad = 0;
+    int rc = tv_validate_queries(vectors, n_new * dim, ix->geo.dim, &bad);   // same predicate, encode.rs:76-83
+    if (rc != TV_OK) {
+        g_last_error = "vector " + std::to_string(bad / dim) + " holds a non-finite or too large value";
+        return rc;
+    }
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    if (ix->n + n_new >= (size_t(1) << 31)) return TV_ERR_BAD_ARGUMENT;
+    rc = ensure_capacity(ix, ix->n + n_new);
+    if (rc != TV_OK) return rc;
+    const size_t slice = std::max<size_t>(1, (size_t(256) << 20) / (dim * sizeof(float)));
+    rc = ensure_workspace(ix, std::min(n_new, slice) * dim * sizeof(float) + 256);
+    if (rc != TV_OK) return rc;
+    for (size_t r0 = 0; r0 < n_new; r0 += slice) {
+        const size_t nr = std::min(slice, n_new - r0);
+        TV_HIP(hipMemcpyAsync(ix->ws, vectors + r0 * dim, nr * dim * sizeof(float), hipMemcpyHostToDevice, ix->stream));
+        rc = add_device_rows(ix, static_cast<const float *>(ix->ws), nr);
+        if (rc != TV_OK) return rc;
+    }
+    return TV_OK;
+}
+
 int tv_index_swap_remove(tv_index *ix, size_t idx) {
     if (!ix) return TV_ERR_BAD_ARGUMENT;
     std::lock_guard<std::mutex> lock(ix->mu);
