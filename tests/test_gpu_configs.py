@@ -1,0 +1,198 @@
+"""Benchmark configurations 3, 4 and 5 at their full sizes, through size-independent
+properties (the oracle cannot finish these in seconds):
+
+  * the rows returned equal an independent ranking of the per-slot scores the
+    scan dumps for the same queries (numpy partition + lexsort, same total order);
+  * sample-then-filter and the exact list/select path agree bit for bit;
+  * top-k of the whole index equals the merge of top-k over a two-way partition
+    of the slots (masks), the reference's split-invariance (search.rs:173-177);
+  * allowlist / mask semantics: every row inside the filter, k_eff = min(k, n_allowed);
+  * planted near-duplicates of database rows come back at rank 1.
+
+Rows are generated on the device (torch) and encoded there (tv_index_add_dev), in
+100k-row chunks as configuration 3 prescribes.
+"""
+import numpy as np
+import pytest
+
+from helpers import bits_equal
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def T():
+    from turbovec_amd import _lib
+    _lib.lib()
+    return _lib
+
+
+def add_generated(ix, n, dim, make_chunk, chunk=100_000):
+    for c0 in range(0, n, chunk):
+        v = make_chunk(c0, min(chunk, n - c0)).contiguous()
+        torch.cuda.synchronize()
+        ix.add_dev(v.data_ptr(), v.shape[0])
+        del v
+
+
+def unit_rows(gen, m, dim):
+    v = torch.randn(m, dim, device="cuda", generator=gen)
+    return v / v.norm(dim=1, keepdim=True)
+
+
+def independent_topk(raw_row, k, allowed=None):
+    """Ranking by (score descending as float compare, slot ascending) without the search path."""
+    sc = raw_row.astype(np.float64)
+    if allowed is not None:
+        sc = np.where(allowed, sc, -np.inf)
+    k = min(k, len(sc))
+    kth = np.partition(sc, len(sc) - k)[len(sc) - k]
+    cand = np.nonzero(sc >= kth)[0]
+    order = cand[np.lexsort((cand, -sc[cand]))][:k]
+    return order
+
+
+def merged(parts, k):
+    s = np.concatenate([p[0] for p in parts], axis=1)
+    i = np.concatenate([p[1] for p in parts], axis=1)
+    out_s, out_i = [], []
+    for r in range(s.shape[0]):
+        o = np.lexsort((i[r], -s[r].astype(np.float64)))[:k]
+        out_s.append(s[r][o]); out_i.append(i[r][o])
+    return np.array(out_s), np.array(out_i)
+
+
+def test_config3_10m_1536_2bit_k100(T):
+    dim, bits, n, k = 1536, 2, 10_000_000, 100
+    gen = torch.Generator(device="cuda"); gen.manual_seed(0)
+    ix = T.NativeIndex(dim, bits)
+    add_generated(ix, n, dim, lambda c0, m: unit_rows(gen, m, dim))
+    assert len(ix) == n
+    qgen = torch.Generator(device="cuda"); qgen.manual_seed(1)
+    q = unit_rows(qgen, 64, dim).cpu().numpy()
+    s, i = ix.search(q, k)
+    assert s.shape == (64, k) and np.all(np.diff(s.astype(np.float64), axis=1) <= 0)
+    assert all(len(set(r.tolist())) == k for r in i)
+    _acc, raw = ix.debug_scan(q[:2])
+    for r in range(2):
+        order = independent_topk(raw[r], k)
+        assert i[r].tolist() == order.tolist() and bits_equal(s[r], raw[r][order])
+    s1, i1 = ix.search(q[3:4], k)                       # batch 1 == its row of the batch
+    assert np.array_equal(i1[0], i[3]) and bits_equal(s1[0], s[3])
+    ix.set_path(1)                                      # exact select path
+    s2, i2 = ix.search(q[:8], k)
+    ix.set_path(0)
+    assert np.array_equal(i2, i[:8]) and bits_equal(s2, s[:8])
+    ix.close()
+
+
+def test_config4_idmap_2m_3072_allowlists():
+    from turbovec_amd import index as api
+    dim, n = 3072, 2_000_000
+    gen = torch.Generator(device="cuda"); gen.manual_seed(0)
+    idx = api.IdMapIndex(dim, 4)
+    rng = np.random.default_rng(0)
+    ids = (rng.permutation(n).astype(np.uint64) * np.uint64(2654435761) + np.uint64(12345))   # unique
+    planted = None
+    for c0 in range(0, n, 100_000):
+        v = unit_rows(gen, 100_000, dim).cpu().numpy()
+        if c0 == 0:
+            planted = v[:64].copy()
+        idx.add_with_ids(v, ids[c0:c0 + 100_000])
+    assert len(idx) == n
+    noise = np.random.default_rng(1).standard_normal(planted.shape).astype(np.float32) * np.float32(0.05 / np.sqrt(dim))
+    q = planted + noise
+    q /= np.linalg.norm(q, axis=1, keepdims=True)
+    s, g = idx.search(q, 10)
+    assert s.shape == (64, 10) and (g[:, 0] == ids[:64]).all()           # each query finds its source row
+    # (a) 1 % of the ids, uniformly at random, the planted rows' ids included for half the queries
+    allow_a = np.concatenate([ids[rng.choice(n, n // 100, replace=False)], ids[:32]])
+    sa, ga = idx.search(q, 10, allowlist=allow_a)
+    aset = set(allow_a.tolist())
+    assert sa.shape == (64, 10) and all(x in aset for x in ga.ravel().tolist())
+    assert (ga[:32, 0] == ids[:32]).all()
+    assert np.all(sa[32:, 0] <= s[32:, 0])
+    # (b) a contiguous 5 % run of insertion order
+    allow_b = ids[1_000_000:1_100_000]
+    sb, gb = idx.search(q, 10, allowlist=allow_b)
+    bset = set(allow_b.tolist())
+    assert sb.shape == (64, 10) and all(x in bset for x in gb.ravel().tolist())
+    # filtered top-k of (a) and (b) both equal the full ranking restricted to the filter where they meet it
+    for r in range(64):
+        in_a = [x for x in g[r].tolist() if x in aset]
+        assert ga[r].tolist()[:len(in_a)] == in_a
+    # (c) sixteen ids, fewer than k=100: rows of exactly sixteen, the same set for every query
+    allow_c = ids[[7, 99, 1234, 50_000, 123_456, 500_000, 999_999, 1_000_000, 1_000_001, 1_500_000,
+                   1_999_999, 31, 32, 33, 64, 0]]
+    sc, gc = idx.search(q, 100, allowlist=allow_c)
+    assert sc.shape == (64, 16) and all(set(r.tolist()) == set(allow_c.tolist()) for r in gc)
+    assert np.all(np.diff(sc.astype(np.float64), axis=1) <= 0)
+    sc10, gc10 = idx.search(q, 10, allowlist=allow_c)
+    assert sc10.shape == (64, 10) and np.array_equal(gc10, gc[:, :10]) and bits_equal(sc10, sc[:, :10])
+    assert (gc[0, 0] == ids[0])                                           # slot 0 is query 0's source
+
+
+def test_config5_10m_1536_clustered_mask_and_churn(T):
+    dim, n, k = 1536, 10_000_000, 10
+    gen = torch.Generator(device="cuda"); gen.manual_seed(0)
+    centres = torch.randn(1000, dim, device="cuda", generator=gen)
+
+    def mixture(m):
+        c = torch.randint(0, 1000, (m,), device="cuda", generator=gen)
+        v = centres[c] + 0.3 * torch.randn(m, dim, device="cuda", generator=gen)
+        return v / v.norm(dim=1, keepdim=True)
+
+    kept = {}
+
+    def chunk(c0, m):
+        v = mixture(m)
+        if c0 == 0:
+            kept["rows"] = v[:1024].clone()
+        return v
+
+    ix = T.NativeIndex(dim, 4)
+    add_generated(ix, n, dim, chunk)
+    qv = kept["rows"] + 0.05 * torch.randn(1024, dim, device="cuda", generator=gen) / (dim ** 0.5)
+    q = (qv / qv.norm(dim=1, keepdim=True)).cpu().numpy()
+    rng = np.random.default_rng(5)
+    m = rng.random(n) < 0.5
+    words, n_allowed = T.pack_mask(m)
+    s, i = ix.search(q, k, mask_words=words)
+    assert s.shape == (1024, k) and m[i].all()
+    src_allowed = m[:1024]
+    assert (i[src_allowed, 0] == np.nonzero(src_allowed)[0]).all()        # allowed sources come back first
+    # exact path and partition merge agree with the sampled path
+    ix.set_path(1)
+    s2, i2 = ix.search(q[:40], k, mask_words=words)
+    ix.set_path(0)
+    assert np.array_equal(i2, i[:40]) and bits_equal(s2, s[:40])
+    wa, _ = T.pack_mask(m & (np.arange(n) % 2 == 0))
+    wb, _ = T.pack_mask(m & (np.arange(n) % 2 == 1))
+    ms, mi = merged([ix.search(q[:64], k, mask_words=wa), ix.search(q[:64], k, mask_words=wb)], k)
+    assert np.array_equal(mi, i[:64]) and bits_equal(ms, s[:64])
+    _acc, raw = ix.debug_scan(q[:2])
+    for r in range(2):
+        order = independent_topk(raw[r], k, allowed=m)
+        assert i[r].tolist() == order.tolist() and bits_equal(s[r], raw[r][order])
+    # churn: remove 1 % of the slots, append 1 % fresh rows; masks are rebuilt afterwards
+    victims = rng.choice(n - 200_000, 100_000, replace=False) + 100_000   # keep the query sources
+    for v in np.sort(victims)[::-1].tolist():
+        ix.swap_remove(v)
+    assert len(ix) == n - 100_000
+    fresh = mixture(100_000).contiguous()
+    torch.cuda.synchronize()
+    ix.add_dev(fresh.data_ptr(), 100_000)
+    assert len(ix) == n
+    s3, i3 = ix.search(q, k)
+    assert (i3[:, 0] == np.arange(1024)).all()
+    m2 = rng.random(n) < 0.5
+    w2, _ = T.pack_mask(m2)
+    s4, i4 = ix.search(q, k, mask_words=w2)
+    assert m2[i4].all()
+    _acc, raw = ix.debug_scan(q[:1])
+    order = independent_topk(raw[0], k, allowed=m2)
+    assert i4[0].tolist() == order.tolist() and bits_equal(s4[0], raw[0][order])
+    order = independent_topk(raw[0], k)
+    assert i3[0].tolist() == order.tolist() and bits_equal(s3[0], raw[0][order])
+    ix.close()
