@@ -343,10 +343,11 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
 
     for (size_t q0 = 0; q0 < nq; q0 += kChunkQueries) {
         const size_t cq = std::min(kChunkQueries, nq - q0);
-        const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_tile_queries(g.nch, 1));
+        const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_append_queries(g.nch));
         const size_t n_tiles = (cq + tile_q - 1) / tile_q;
         const size_t cq_pad = n_tiles * tile_q;
-        const int grid = tv::scan_grid_blocks(ix->device, mode_p, g.nch, 0, int(tile_q));
+        const int grid = mode_p ? tv::scan_grid_blocks(ix->device, mode_p, g.nch, 0, int(tile_q))
+                                : tv::lut_append_grid(ix->device, g.nch);
         const size_t seg_stride = size_t(grid);
         size_t need = prepare_bytes(ix, cq) + round_up(n_tiles * tv::kQTile * 4, 256) +
                       round_up(cq_pad * seg_stride * tv::kSegCap * 8, 256) + round_up(cq_pad * seg_stride * 4, 256) +

@@ -97,6 +97,8 @@ size_t scan_lds_bytes(int mode_p, int nch, int k, int lut_queries);
 int lut_tile_queries(int nch, int k);
 // Queries per LDS entry (1, 2 or 4) the LUT scan launch picks for nq_tile queries.
 int lut_launch_ql(int nch, int k, int nq_tile);
+int lut_append_queries(int nch);
+int lut_append_grid(int device, int nch);
 hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s);
 hipError_t launch_scan_lut(const ScanArgs &a, int grid, int mode, hipStream_t s);
 // Query tiles one batched permute-dot launch serves for this geometry (0: not available).

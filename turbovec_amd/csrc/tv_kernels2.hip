@@ -12,33 +12,73 @@ namespace tv {
 // (turbovec/src/search.rs:3113-3128 is the definition; the production kernels
 // are :467-670, :697-984, :1071-1339).  QL queries share one pass: their
 // tables are interleaved entry-major in LDS so that one QL-byte LDS read
-// fetches the same entry of all QL queries, and the bytes are accumulated as
-// packed 16-bit lanes that are widened every 256 byte-groups -- the same flush
-// period the reference uses, which makes the classic epilogue's per-batch
-// fma(scale, f32(batch_sum), fa) reproducible exactly.
+// fetches the same entry of all QL queries.  The two reads of a code byte are
+// added bytewise (entries are at most 127, so no byte carries) and each
+// query's byte is peeled into its own 32-bit sum with one v_dot4_u32_u8
+// against a one-hot constant.  Sums are flushed every 256 byte-groups -- the
+// reference's period -- which makes the classic epilogue's per-batch
+// fma(scale, f32(batch_sum), fa) reproducible exactly.  Append-mode launches
+// use 1024-thread workgroups: one copy of the tables in LDS then serves four
+// waves per SIMD, which is what hides the LDS and HBM latencies.
 // ===========================================================================
 
 template <int QL> struct LutWord;
 template <> struct LutWord<1> { typedef uint8_t type; };
 template <> struct LutWord<2> { typedef uint16_t type; };
 template <> struct LutWord<4> { typedef uint32_t type; };
+template <> struct LutWord<8> { typedef uint2 type; };
 
-template <int QL, int U, int MODE, bool LUT_LDS>
-__global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
+// acc[q] += byte q of (vh + vl), bytewise sums never carrying (entries <= 127).
+template <int QL> struct LutAcc;
+template <> struct LutAcc<1> {
+    static __device__ __forceinline__ void add(uint32_t (&acc)[1], uint8_t vh, uint8_t vl) { acc[0] += uint32_t(vh) + uint32_t(vl); }
+};
+template <> struct LutAcc<2> {
+    static __device__ __forceinline__ void add(uint32_t (&acc)[2], uint16_t vh, uint16_t vl) {
+        const uint32_t s = uint32_t(vh) + uint32_t(vl);
+        acc[0] = __builtin_amdgcn_udot4(s, 0x00000001u, acc[0], false);
+        acc[1] = __builtin_amdgcn_udot4(s, 0x00000100u, acc[1], false);
+    }
+};
+template <> struct LutAcc<4> {
+    static __device__ __forceinline__ void add(uint32_t (&acc)[4], uint32_t vh, uint32_t vl) {
+        const uint32_t s = vh + vl;
+        acc[0] = __builtin_amdgcn_udot4(s, 0x00000001u, acc[0], false);
+        acc[1] = __builtin_amdgcn_udot4(s, 0x00000100u, acc[1], false);
+        acc[2] = __builtin_amdgcn_udot4(s, 0x00010000u, acc[2], false);
+        acc[3] = __builtin_amdgcn_udot4(s, 0x01000000u, acc[3], false);
+    }
+};
+template <> struct LutAcc<8> {
+    static __device__ __forceinline__ void add(uint32_t (&acc)[8], uint2 vh, uint2 vl) {
+        const uint32_t s0 = vh.x + vl.x, s1 = vh.y + vl.y;
+        acc[0] = __builtin_amdgcn_udot4(s0, 0x00000001u, acc[0], false);
+        acc[1] = __builtin_amdgcn_udot4(s0, 0x00000100u, acc[1], false);
+        acc[2] = __builtin_amdgcn_udot4(s0, 0x00010000u, acc[2], false);
+        acc[3] = __builtin_amdgcn_udot4(s0, 0x01000000u, acc[3], false);
+        acc[4] = __builtin_amdgcn_udot4(s1, 0x00000001u, acc[4], false);
+        acc[5] = __builtin_amdgcn_udot4(s1, 0x00000100u, acc[5], false);
+        acc[6] = __builtin_amdgcn_udot4(s1, 0x00010000u, acc[6], false);
+        acc[7] = __builtin_amdgcn_udot4(s1, 0x01000000u, acc[7], false);
+    }
+};
+
+template <int QL, int U, int MODE, bool LUT_LDS, int THREADS>
+__global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
     typedef typename LutWord<QL>::type word_t;
     constexpr bool LISTS = MODE == kModeLists, DUMP = MODE == kModeDump, APPEND = MODE == kModeAppend;
     extern __shared__ __align__(16) uint8_t smem[];
     const int nch = a.nch, k = a.k;
     const size_t lut_bytes = LUT_LDS ? size_t(nch) * 1024 * QL : 0;
-    float *sct = reinterpret_cast<float *>(smem + lut_bytes);            // [4 waves][QL][32]
-    float *ls = sct + 4 * QL * 32;
-    uint32_t *li = reinterpret_cast<uint32_t *>(ls + (LISTS ? k * kScanThreads : 0));
-    int *stau = reinterpret_cast<int *>(li + (LISTS ? k * kScanThreads : 0));
+    float *sct = reinterpret_cast<float *>(smem + lut_bytes);            // [waves][QL][32]
+    float *ls = sct + (THREADS / 64) * QL * 32;
+    uint32_t *li = reinterpret_cast<uint32_t *>(ls + (LISTS ? k * THREADS : 0));
+    int *stau = reinterpret_cast<int *>(li + (LISTS ? k * THREADS : 0));
     const int tid = threadIdx.x;
 
     if (LUT_LDS) {
         // interleave: entry e of query qq -> smem[e*QL + qq]
-        for (int w = tid; w < nch * 256; w += kScanThreads) {
+        for (int w = tid; w < nch * 256; w += THREADS) {
             uint32_t v[QL];
 #pragma unroll
             for (int qq = 0; qq < QL; ++qq)
@@ -72,7 +112,7 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
 
     const uint32_t step = a.b_step;
     const uint32_t nj = (a.n_blocks + step - 1) / step;
-    const uint32_t total_waves = gridDim.x * (kScanThreads / 64);
+    const uint32_t total_waves = gridDim.x * (THREADS / 64);
     const uint32_t gw = wave * gridDim.x + blockIdx.x;  // consecutive blocks go to different workgroups
     const uint32_t j_begin = gw, j_end = nj;   // round-robin over the grid's waves
 
@@ -104,7 +144,9 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
         float fa[QL];
 #pragma unroll
         for (int qq = 0; qq < QL; ++qq) { total[qq] = 0; fa[qq] = qb[qq]; }
-        uint32_t accE = 0, accO = 0;
+        uint32_t acc[QL];
+#pragma unroll
+        for (int qq = 0; qq < QL; ++qq) acc[qq] = 0;
         for (int c0 = 0; c0 < nch; c0 += U) {
             uint4 cur[U];
 #pragma unroll
@@ -120,31 +162,21 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
             for (int u = 0; u < U; ++u) {
                 const int c = c0 + u;
                 const uint32_t x[4] = {cur[u].x, cur[u].y, cur[u].z, cur[u].w};
-                const int g0 = c * 32 + 16 * h;
+                const word_t *rowp = lut + (c * 32 + 16 * h) * 32;
 #pragma unroll
                 for (int j = 0; j < 16; ++j) {
                     const uint32_t byte = (x[j >> 2] >> (8 * (j & 3))) & 0xffu;
-                    const int row = (g0 + j) * 32;
-                    const uint32_t vh = lut[row + (byte >> 4)];
-                    const uint32_t vl = lut[row + 16 + (byte & 15u)];
-                    if (QL == 1) {
-                        accE += vh + vl;
-                    } else {
-                        accE += (vh & 0x00ff00ffu) + (vl & 0x00ff00ffu);
-                        accO += ((vh >> 8) & 0x00ff00ffu) + ((vl >> 8) & 0x00ff00ffu);
-                    }
+                    const word_t vh = rowp[j * 32 + (byte >> 4)];
+                    const word_t vl = rowp[j * 32 + 16 + (byte & 15u)];
+                    LutAcc<QL>::add(acc, vh, vl);
                 }
                 if ((c & 7) == 7 || c == nch - 1) {  // end of a 256-group batch (search.rs:529-531)
-                    uint32_t part[QL];
-                    if (QL == 1) part[0] = accE;
-                    if (QL == 2) { part[0] = accE; part[1] = accO; }
-                    if (QL == 4) { part[0] = accE & 0xffffu; part[1] = accO & 0xffffu; part[2] = accE >> 16; part[3] = accO >> 16; }
-                    accE = 0; accO = 0;
 #pragma unroll
                     for (int qq = 0; qq < QL; ++qq) {
-                        part[qq] += __shfl_xor(int(part[qq]), 32);
-                        total[qq] += part[qq];
-                        fa[qq] = fmaf(qs[qq], float(part[qq]), fa[qq]);  // search.rs:577-580
+                        const uint32_t part = acc[qq] + uint32_t(__shfl_xor(int(acc[qq]), 32));
+                        acc[qq] = 0;
+                        total[qq] += part;
+                        fa[qq] = fmaf(qs[qq], float(part), fa[qq]);  // search.rs:577-580
                     }
                 }
             }
@@ -202,7 +234,7 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
                         const uint32_t slot = slot0 + i;
                         if (s >= tau && (L.cnt < k || ranks_before(s, slot, L.worst_s, L.worst_i))) {
                             if (slot < a.n && ((mw >> i) & 1u)) {
-                                if (list_offer(L, ls, li, kScanThreads, tid, k, s, slot) && a.share_tau) {
+                                if (list_offer(L, ls, li, THREADS, tid, k, s, slot) && a.share_tau) {
                                     const int key = order_key(L.worst_s);
                                     if (atomicMax(&stau[oq], key) < key) atomicMax(&a.gtau[oq], key);
                                 }
@@ -222,27 +254,47 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_lut(ScanArgs a) {
         if (tid < a.nq_tile) a.cand_cnt[size_t(tid) * a.seg_stride + blockIdx.x] = scnt[tid];
     }
     if (LISTS) {
-        const size_t total_threads = size_t(gridDim.x) * kScanThreads;
-        const size_t gt = size_t(blockIdx.x) * kScanThreads + tid;
+        const size_t total_threads = size_t(gridDim.x) * THREADS;
+        const size_t gt = size_t(blockIdx.x) * THREADS + tid;
         a.part_cnt[gt] = L.cnt;
         for (int e = 0; e < L.cnt; ++e) {
-            a.part_scores[size_t(e) * total_threads + gt] = ls[e * kScanThreads + tid];
-            a.part_idx[size_t(e) * total_threads + gt] = li[e * kScanThreads + tid];
+            a.part_scores[size_t(e) * total_threads + gt] = ls[e * THREADS + tid];
+            a.part_idx[size_t(e) * total_threads + gt] = li[e * THREADS + tid];
         }
     }
 }
 
 static constexpr size_t kLdsBudgetL = 160 * 1024;
 
-static size_t lut_lds_bytes(int nch, int k, int ql, bool no_lists) {
-    const size_t lists = no_lists ? 0 : size_t(k) * kScanThreads * 8;
-    return size_t(nch) * 1024 * ql + size_t(4) * ql * 32 * 4 + lists + kQTile * sizeof(int);
+static size_t lut_lds_bytes(int nch, int k, int ql, bool no_lists, int threads) {
+    const size_t lists = no_lists ? 0 : size_t(k) * threads * 8;
+    return size_t(nch) * 1024 * ql + size_t(threads / 64) * ql * 32 * 4 + lists + kQTile * sizeof(int);
 }
 
+constexpr int kLutListThreads = kScanThreads;   // exact paths: per-lane lists or dense dump
+constexpr int kLutAppendThreads = 1024;         // sample-then-filter scans
+
+// Queries one list- or dump-mode launch serves.
 int lut_tile_queries(int nch, int k) {
     for (int ql = 4; ql >= 1; ql >>= 1)
-        if (lut_lds_bytes(nch, k, ql, false) <= kLdsBudgetL) return ql;
+        if (lut_lds_bytes(nch, k, ql, false, kLutListThreads) <= kLdsBudgetL) return ql;
     return 1;  // table read from global memory
+}
+
+// Queries one append-mode launch serves (tables of all of them resident in LDS, one copy per CU).
+int lut_append_queries(int nch) {
+    for (int ql = 8; ql >= 1; ql >>= 1)
+        if (lut_lds_bytes(nch, 0, ql, true, kLutAppendThreads) <= kLdsBudgetL) return ql;
+    return 1;
+}
+
+int lut_append_grid(int device, int nch) {
+    hipDeviceProp_t prop;
+    int cus = 256;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0)
+        cus = prop.multiProcessorCount;
+    const size_t lds = lut_lds_bytes(nch, 0, lut_append_queries(nch), true, kLutAppendThreads);
+    return cus * (lds * 2 <= kLdsBudgetL ? 2 : 1);   // at most 2048 threads per CU
 }
 
 template <typename K>
@@ -258,31 +310,39 @@ int lut_launch_ql(int nch, int k, int nq_tile) {
     return ql;
 }
 
-// One launch serves a.nq_tile <= lut_tile_queries(nch, k) queries.
+// One launch serves a.nq_tile queries: at most lut_append_queries(nch) in append mode,
+// lut_tile_queries(nch, k) otherwise.
 hipError_t launch_scan_lut(const ScanArgs &a, int grid, int mode, hipStream_t s) {
+    const bool append = mode == kModeAppend;
     const bool dump = mode != kModeLists;   // no list storage in LDS
     const int kk = a.k;                     // the tile width is chosen for the list pass of the same search
-    const int ql = lut_launch_ql(a.nch, kk, a.nq_tile);
-    const bool in_lds = lut_lds_bytes(a.nch, kk, ql, dump) <= kLdsBudgetL;
-    const size_t lds = in_lds ? lut_lds_bytes(a.nch, kk, ql, dump)
-                              : lut_lds_bytes(0, kk, 1, dump);
+    const int threads = append ? kLutAppendThreads : kLutListThreads;
+    int ql = append ? lut_append_queries(a.nch) : lut_tile_queries(a.nch, kk);
+    while (ql > 1 && ql / 2 >= a.nq_tile) ql >>= 1;
+    const bool in_lds = lut_lds_bytes(a.nch, kk, ql, dump, threads) <= kLdsBudgetL;
+    const size_t lds = in_lds ? lut_lds_bytes(a.nch, kk, ql, dump, threads)
+                              : lut_lds_bytes(0, kk, 1, dump, threads);
     hipError_t e = hipSuccess;
-#define TV_LAUNCH_L(QL, U, D, W)                                                                 \
+#define TV_LAUNCH_L(QL, U, D, W, T)                                                              \
     do {                                                                                         \
-        e = allow_lds2(k_scan_lut<QL, U, D, W>, lds);                                            \
+        e = allow_lds2(k_scan_lut<QL, U, D, W, T>, lds);                                         \
         if (e != hipSuccess) return e;                                                           \
-        hipLaunchKernelGGL((k_scan_lut<QL, U, D, W>), dim3(grid), dim3(kScanThreads), lds, s, a); \
+        hipLaunchKernelGGL((k_scan_lut<QL, U, D, W, T>), dim3(grid), dim3(T), lds, s, a);        \
     } while (0)
 #define TV_PICK_M(QL, U, W)                                                                      \
     do {                                                                                         \
-        if (mode == kModeDump) TV_LAUNCH_L(QL, U, kModeDump, W);                                 \
-        else if (mode == kModeAppend) TV_LAUNCH_L(QL, U, kModeAppend, W);                        \
-        else TV_LAUNCH_L(QL, U, kModeLists, W);                                                  \
+        if (mode == kModeDump) TV_LAUNCH_L(QL, U, kModeDump, W, kLutListThreads);                \
+        else if (mode == kModeAppend) TV_LAUNCH_L(QL, U, kModeAppend, W, kLutAppendThreads);     \
+        else TV_LAUNCH_L(QL, U, kModeLists, W, kLutListThreads);                                 \
     } while (0)
 #define TV_PICK_L(QL, U) TV_PICK_M(QL, U, true)
     const int u = a.nch % 2 == 0 ? 2 : 1;
     if (!in_lds) {
         if (u == 2) TV_PICK_M(1, 2, false); else TV_PICK_M(1, 1, false);
+    } else if (ql == 8) {
+        if (!append) return hipErrorInvalidValue;
+        if (u == 2) TV_LAUNCH_L(8, 2, kModeAppend, true, kLutAppendThreads);
+        else TV_LAUNCH_L(8, 1, kModeAppend, true, kLutAppendThreads);
     } else if (ql == 4) { if (u == 2) TV_PICK_L(4, 2); else TV_PICK_L(4, 1); }
     else if (ql == 2) { if (u == 2) TV_PICK_L(2, 2); else TV_PICK_L(2, 1); }
     else { if (u == 2) TV_PICK_L(1, 2); else TV_PICK_L(1, 1); }
