@@ -22,11 +22,27 @@ namespace tv {
 // waves per SIMD, which is what hides the LDS and HBM latencies.
 // ===========================================================================
 
+// base + byte E of packed, in one instruction (sub-dword operand select).
+template <int E>
+__device__ __forceinline__ uint32_t add_byte(uint32_t base, uint32_t packed) {
+    uint32_t r;
+    if (E == 0) asm("v_add_u32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0" : "=v"(r) : "v"(base), "v"(packed));
+    if (E == 1) asm("v_add_u32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1" : "=v"(r) : "v"(base), "v"(packed));
+    if (E == 2) asm("v_add_u32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2" : "=v"(r) : "v"(base), "v"(packed));
+    if (E == 3) asm("v_add_u32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3" : "=v"(r) : "v"(base), "v"(packed));
+    return r;
+}
+
+template <int V> struct IntC { static constexpr int value = V; };
+template <typename F>
+__device__ __forceinline__ void static_for4(F &&f) { f(IntC<0>{}); f(IntC<1>{}); f(IntC<2>{}); f(IntC<3>{}); }
+
 template <int QL> struct LutWord;
 template <> struct LutWord<1> { typedef uint8_t type; };
 template <> struct LutWord<2> { typedef uint16_t type; };
 template <> struct LutWord<4> { typedef uint32_t type; };
-template <> struct LutWord<8> { typedef uint2 type; };
+typedef uint32_t lut_u32x2 __attribute__((ext_vector_type(2)));
+template <> struct LutWord<8> { typedef lut_u32x2 type; };
 
 // acc[q] += byte q of (vh + vl), bytewise sums never carrying (entries <= 127).
 template <int QL> struct LutAcc;
@@ -50,7 +66,7 @@ template <> struct LutAcc<4> {
     }
 };
 template <> struct LutAcc<8> {
-    static __device__ __forceinline__ void add(uint32_t (&acc)[8], uint2 vh, uint2 vl) {
+    static __device__ __forceinline__ void add(uint32_t (&acc)[8], lut_u32x2 vh, lut_u32x2 vl) {
         const uint32_t s0 = vh.x + vl.x, s1 = vh.y + vl.y;
         acc[0] = __builtin_amdgcn_udot4(s0, 0x00000001u, acc[0], false);
         acc[1] = __builtin_amdgcn_udot4(s0, 0x00000100u, acc[1], false);
@@ -95,6 +111,10 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
     if (APPEND && tid < kQTile) scnt[tid] = 0u;
     __syncthreads();
     const word_t *lut = LUT_LDS ? reinterpret_cast<const word_t *>(smem) : reinterpret_cast<const word_t *>(a.tables);
+    // the tables' address inside LDS as a plain number: entry addresses are then formed with integer
+    // adds and dereferenced as LDS pointers, with the per-byte row offsets riding in the read's offset field
+    typedef const __attribute__((address_space(3))) word_t lds_word_t;
+    const uint32_t lds_lut_addr = uint32_t(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)smem));
 
     const int lane = tid & 63, wave = tid >> 6;
     const int vi = lane & 31, h = lane >> 5;
@@ -162,13 +182,29 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
             for (int u = 0; u < U; ++u) {
                 const int c = c0 + u;
                 const uint32_t x[4] = {cur[u].x, cur[u].y, cur[u].z, cur[u].w};
-                const word_t *rowp = lut + (c * 32 + 16 * h) * 32;
+                // Byte offsets of the entries inside their 16-entry sub-tables, four code bytes at a
+                // time: nibble * sizeof(word) still fits a byte, so one shift and one mask prepare
+                // four of them and a byte-select add forms each LDS address.
+                constexpr int kSh = QL == 1 ? 0 : QL == 2 ? 1 : QL == 4 ? 2 : 3;
+                const uint8_t *gbase = reinterpret_cast<const uint8_t *>(lut);
+                const uint32_t row_off = uint32_t(c * 32 + 16 * h) * 32 * QL + (LUT_LDS ? lds_lut_addr : 0u);
 #pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    const uint32_t byte = (x[j >> 2] >> (8 * (j & 3))) & 0xffu;
-                    const word_t vh = rowp[j * 32 + (byte >> 4)];
-                    const word_t vl = rowp[j * 32 + 16 + (byte & 15u)];
-                    LutAcc<QL>::add(acc, vh, vl);
+                for (int d = 0; d < 4; ++d) {
+                    const uint32_t plo = (x[d] << kSh) & (0x0f0f0f0fu << kSh);
+                    const uint32_t phi = (x[d] >> (4 - kSh)) & (0x0f0f0f0fu << kSh);
+                    static_for4([&](auto ec) {
+                        constexpr int e = decltype(ec)::value;
+                        const int j = d * 4 + e;
+                        word_t vh, vl;
+                        if (LUT_LDS) {
+                            vh = *reinterpret_cast<lds_word_t *>(add_byte<e>(row_off, phi) + j * 32 * QL);
+                            vl = *reinterpret_cast<lds_word_t *>(add_byte<e>(row_off, plo) + (j * 32 + 16) * QL);
+                        } else {
+                            vh = *reinterpret_cast<const word_t *>(gbase + add_byte<e>(row_off, phi) + j * 32 * QL);
+                            vl = *reinterpret_cast<const word_t *>(gbase + add_byte<e>(row_off, plo) + (j * 32 + 16) * QL);
+                        }
+                        LutAcc<QL>::add(acc, vh, vl);
+                    });
                 }
                 if ((c & 7) == 7 || c == nch - 1) {  // end of a 256-group batch (search.rs:529-531)
 #pragma unroll
