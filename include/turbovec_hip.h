@@ -40,7 +40,8 @@ typedef enum {
     TV_ERR_BAD_ARGUMENT = 6,                     /* ConstructError / FromPartsError class */
     TV_ERR_HIP = 7,                              /* a HIP runtime call failed */
     TV_ERR_NO_DEVICE = 8,                        /* no gfx950 device visible */
-    TV_ERR_INDEX_OUT_OF_RANGE = 9
+    TV_ERR_INDEX_OUT_OF_RANGE = 9,
+    TV_ERR_BAD_IMAGE = 10        /* snapshot bytes refused; tv_last_error says why */
 } tv_status;
 
 /* Which integer score definition the scan uses (the reference picks one at run
@@ -139,6 +140,37 @@ int tv_search_dev(tv_index *ix, const float *d_queries, size_t nq, size_t k,
  * signs/perms 2*dim each, round 0 first) and codebook::codebook (codebook.rs:50). */
 int tv_host_rotation_tables(int dim, float *signs, uint32_t *perms, int *block, float *inv_sqrt_block);
 int tv_host_codebook(int bits, int dim, float *boundaries, float *centroids);
+
+/* ---- snapshot images (turbovec/src/io_v7.rs) ------------------------------- */
+
+/* The byte form TurboQuantIndex::to_bytes (lib.rs:2167) / IdMapIndex::to_bytes
+ * (id_map.rs:971) and `write` produce: an unclaimed generation-0 TV7 image
+ * (io_v7.rs:902-925 write_image: superblock :516-542, header slot :549-599,
+ * units :602-629, CRC-32C :128-141).  kind 0 = slot-addressed index, 1 = id map.
+ * format 7 is that image; format 6 is the flat TVPI / TVIM container of the
+ * release before (convert.rs:14-31, :453-512), which the reference's committed
+ * sha256 digests of to_bytes() still hash.  These four touch no GPU. */
+size_t tv_host_snapshot_len(int format, int dim, int bits, int kind, size_t n_calib, size_t n);
+/* seq: sequential-blocked codes of n rows (what tv_index_download_seq returns);
+ * shift/scale: n_calib floats each (n_calib is 0 or dim); ids: n values, kind 1 only.
+ * out must hold tv_host_snapshot_len(...) bytes. */
+int tv_host_snapshot_compose(int format, int dim, int bits, int kind, const float *boundaries, const float *centroids,
+                             size_t n_calib, const float *shift, const float *scale,
+                             const uint8_t *seq, size_t n, const float *scales, const uint64_t *ids,
+                             uint8_t *out);
+/* Validate an image of either format (magic, revision, checksums, geometry, that a TV7
+ * image is a snapshot and not a synced container with pending operations) and report its shape. */
+int tv_host_snapshot_info(const uint8_t *bytes, size_t len, int *format, int *kind, int *dim, int *bits,
+                          size_t *n_calib, size_t *n);
+/* Unpack a validated image; any output pointer may be NULL.  seq: ceil(n/32)*G*32 bytes. */
+int tv_host_snapshot_extract(const uint8_t *bytes, size_t len, float *boundaries, float *centroids,
+                             float *shift, float *scale, uint8_t *seq, float *scales, uint64_t *ids);
+/* Snapshot of a device-resident index.  ids == NULL writes kind 0, otherwise kind 1 with
+ * ids[slot] (id_map.rs slot_to_id).  out == NULL only reports *len. */
+int tv_index_to_bytes(const tv_index *ix, const uint64_t *ids, int format, uint8_t *out, size_t cap, size_t *len);
+/* Build a device-resident index from an image (replaces from_v7_image, lib.rs:2196);
+ * ids_out (may be NULL) receives n ids for a kind-1 image. */
+int tv_index_from_bytes(const uint8_t *bytes, size_t len, int device, tv_index **out, uint64_t *ids_out);
 
 /* ---- test / measurement hooks -------------------------------------------- */
 

@@ -31,6 +31,8 @@ EXPORTS = [
     "tv_index_bits", "tv_validate_queries", "tv_pack_mask", "tv_search", "tv_search_dev", "tv_debug_scan",
     "tv_debug_prepare", "tv_last_scan_ms", "tv_index_device_ptrs", "tv_host_rotation_tables", "tv_host_codebook",
     "tv_debug_stream_probe", "tv_debug_set_path", "tv_debug_overflow_redos",
+    "tv_host_snapshot_len", "tv_host_snapshot_compose", "tv_host_snapshot_info", "tv_host_snapshot_extract",
+    "tv_index_to_bytes", "tv_index_from_bytes",
 ]
 
 _lib = None
@@ -66,6 +68,13 @@ def lib():
     L.tv_index_upload_seq_dev.argtypes = [vp, vp, sz, vp]
     L.tv_index_append_rows.argtypes = [vp, vp, vp, sz]
     L.tv_index_add.argtypes = [vp, vp, sz]
+    L.tv_host_snapshot_len.restype = sz
+    L.tv_host_snapshot_len.argtypes = [i32, i32, i32, i32, sz, sz]
+    L.tv_host_snapshot_compose.argtypes = [i32, i32, i32, i32, vp, vp, sz, vp, vp, vp, sz, vp, vp, vp]
+    L.tv_host_snapshot_info.argtypes = [vp, sz, C.POINTER(i32), C.POINTER(i32), C.POINTER(i32), C.POINTER(i32), C.POINTER(sz), C.POINTER(sz)]
+    L.tv_host_snapshot_extract.argtypes = [vp, sz, vp, vp, vp, vp, vp, vp, vp]
+    L.tv_index_to_bytes.argtypes = [vp, vp, i32, vp, sz, C.POINTER(sz)]
+    L.tv_index_from_bytes.argtypes = [vp, sz, i32, C.POINTER(vp), vp]
     L.tv_index_add_dev.argtypes = [vp, vp, sz]
     L.tv_index_swap_remove.argtypes = [vp, sz]
     L.tv_index_download_seq.argtypes = [vp, vp, vp]
@@ -175,6 +184,33 @@ class NativeIndex:
     def swap_remove(self, idx):
         check(lib().tv_index_swap_remove(self.h, idx))
 
+    def to_bytes(self, ids=None, format=7):
+        """Snapshot image (tv_index_to_bytes); ids (uint64, one per slot) makes it an id-map image."""
+        idp = None
+        if ids is not None:
+            ids = np.ascontiguousarray(ids, np.uint64)
+            assert len(ids) == len(self)
+            idp = ptr(ids)
+        n = C.c_size_t(0)
+        check(lib().tv_index_to_bytes(self.h, idp, format, None, 0, C.byref(n)))
+        out = np.zeros(n.value, np.uint8)
+        check(lib().tv_index_to_bytes(self.h, idp, format, ptr(out), n.value, C.byref(n)))
+        return out.tobytes()
+
+    @classmethod
+    def from_bytes(cls, data, device=0):
+        """(index, ids or None) from a snapshot image (tv_index_from_bytes)."""
+        _fmt, kind, dim, bits, n_calib, n = snapshot_info(data)
+        buf = np.frombuffer(data, np.uint8)
+        ids = np.zeros(n, np.uint64) if kind == 1 else None
+        h = C.c_void_p()
+        check(lib().tv_index_from_bytes(ptr(buf), len(buf), device, C.byref(h), ptr(ids) if ids is not None else None))
+        self = cls.__new__(cls)
+        self.h = h
+        self.dim, self.bits = dim, bits
+        self.n_byte_groups = dim // (4 if bits == 2 else 2)
+        return self, ids
+
     def download_seq(self):
         n = len(self)
         seq = np.zeros(((n + 31) // 32) * self.n_byte_groups * 32, np.uint8)
@@ -260,6 +296,57 @@ def pack_mask(mask_bytes):
     allowed = C.c_size_t(0)
     check(lib().tv_pack_mask(ptr(m), m.size, ptr(words), C.byref(allowed)))
     return words, allowed.value
+
+
+def snapshot_info(data):
+    buf = np.frombuffer(data, np.uint8)
+    fmt, kind, dim, bits = C.c_int(0), C.c_int(0), C.c_int(0), C.c_int(0)
+    n_calib, n = C.c_size_t(0), C.c_size_t(0)
+    check(lib().tv_host_snapshot_info(ptr(buf), len(buf), C.byref(fmt), C.byref(kind), C.byref(dim), C.byref(bits),
+                                      C.byref(n_calib), C.byref(n)))
+    return fmt.value, kind.value, dim.value, bits.value, n_calib.value, n.value
+
+
+def snapshot_compose(dim, bits, boundaries, centroids, seq, n, scales, calibration=None, ids=None, format=7):
+    """Host-only: the snapshot image of an index given in the persisted layout."""
+    kind = 0 if ids is None else 1
+    b = np.ascontiguousarray(boundaries, np.float32)
+    c = np.ascontiguousarray(centroids, np.float32)
+    sh = sc = None
+    n_calib = 0
+    if calibration is not None:
+        sh = np.ascontiguousarray(calibration[0], np.float32)
+        sc = np.ascontiguousarray(calibration[1], np.float32)
+        n_calib = len(sh)
+    seq = np.ascontiguousarray(seq, np.uint8)
+    scales = np.ascontiguousarray(scales, np.float32)
+    if ids is not None:
+        ids = np.ascontiguousarray(ids, np.uint64)
+    out = np.zeros(lib().tv_host_snapshot_len(format, dim, bits, kind, n_calib, n), np.uint8)
+    check(lib().tv_host_snapshot_compose(format, dim, bits, kind, ptr(b), ptr(c), n_calib,
+                                         ptr(sh) if sh is not None else None, ptr(sc) if sc is not None else None,
+                                         ptr(seq) if n else None, n, ptr(scales) if n else None,
+                                         ptr(ids) if ids is not None and n else None, ptr(out)))
+    return out.tobytes()
+
+
+def snapshot_extract(data):
+    """Host-only: (dict of arrays) unpacked from a snapshot image."""
+    fmt, kind, dim, bits, n_calib, n = snapshot_info(data)
+    buf = np.frombuffer(data, np.uint8)
+    G = dim // (4 if bits == 2 else 2)
+    nl = 1 << bits
+    out = dict(format=fmt, kind=kind, dim=dim, bits=bits, n=n,
+               boundaries=np.zeros(nl - 1, np.float32), centroids=np.zeros(nl, np.float32),
+               shift=np.zeros(n_calib, np.float32), scale=np.zeros(n_calib, np.float32),
+               seq=np.zeros(((n + 31) // 32) * G * 32, np.uint8), scales=np.zeros(((n + 31) // 32) * 32, np.float32),
+               ids=np.zeros(((n + 31) // 32) * 32, np.uint64))
+    check(lib().tv_host_snapshot_extract(ptr(buf), len(buf), ptr(out["boundaries"]), ptr(out["centroids"]),
+                                         ptr(out["shift"]), ptr(out["scale"]), ptr(out["seq"]), ptr(out["scales"]),
+                                         ptr(out["ids"])))
+    out["scales"] = out["scales"][:n]
+    out["ids"] = out["ids"][:n] if kind == 1 else None
+    return out
 
 
 def host_rotation_tables(dim):

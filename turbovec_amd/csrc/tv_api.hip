@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "tv_internal.h"
+#include "tv_snapshot.h"
 
 namespace {
 
@@ -449,6 +450,7 @@ const char *tv_status_string(int status) {
         case TV_ERR_HIP: return "HIP runtime error";
         case TV_ERR_NO_DEVICE: return "no usable GPU";
         case TV_ERR_INDEX_OUT_OF_RANGE: return "index out of range";
+        case TV_ERR_BAD_IMAGE: return "invalid snapshot image";
         default: return "unknown status";
     }
 }
@@ -908,6 +910,107 @@ int tv_host_codebook(int bits, int dim, float *boundaries, float *centroids) {
     const tv::Codebook cb = tv::make_codebook(bits, dim);
     if (boundaries) std::memcpy(boundaries, cb.boundaries.data(), cb.boundaries.size() * sizeof(float));
     if (centroids) std::memcpy(centroids, cb.centroids.data(), cb.centroids.size() * sizeof(float));
+    return TV_OK;
+}
+
+size_t tv_host_snapshot_len(int format, int dim, int bits, int kind, size_t n_calib, size_t n) {
+    if (format != 6 && format != 7) return 0;
+    return tv::snapshot_len(format, dim, bits, kind, n_calib, n);
+}
+
+int tv_host_snapshot_compose(int format, int dim, int bits, int kind, const float *boundaries, const float *centroids,
+                             size_t n_calib, const float *shift, const float *scale,
+                             const uint8_t *seq, size_t n, const float *scales, const uint64_t *ids,
+                             uint8_t *out) {
+    if (format != 6 && format != 7) return TV_ERR_BAD_ARGUMENT;
+    if (bits < 2 || bits > 4 || dim <= 0 || dim % 8 != 0 || dim > 16384 || kind < 0 || kind > 1) return TV_ERR_BAD_ARGUMENT;
+    if (!boundaries || !centroids || !out || (n && (!seq || !scales)) || (kind == 1 && n && !ids)) return TV_ERR_BAD_ARGUMENT;
+    if ((n_calib != 0 && n_calib != size_t(dim)) || (n_calib && (!shift || !scale))) return TV_ERR_BAD_ARGUMENT;
+    const tv::SnapshotParts s{kind, dim, bits, boundaries, centroids, n_calib, shift, scale, seq, n, scales, ids};
+    tv::snapshot_compose(format, s, out);
+    return TV_OK;
+}
+
+int tv_host_snapshot_info(const uint8_t *bytes, size_t len, int *format, int *kind, int *dim, int *bits,
+                          size_t *n_calib, size_t *n) {
+    if (!bytes) return TV_ERR_BAD_ARGUMENT;
+    tv::SnapshotInfo info;
+    const std::string why = tv::snapshot_parse(bytes, len, info);
+    if (!why.empty()) { g_last_error = why; return TV_ERR_BAD_IMAGE; }
+    if (format) *format = info.format;
+    if (kind) *kind = info.kind;
+    if (dim) *dim = info.dim;
+    if (bits) *bits = info.bits;
+    if (n_calib) *n_calib = info.n_calib;
+    if (n) *n = info.n;
+    return TV_OK;
+}
+
+int tv_host_snapshot_extract(const uint8_t *bytes, size_t len, float *boundaries, float *centroids,
+                             float *shift, float *scale, uint8_t *seq, float *scales, uint64_t *ids) {
+    if (!bytes) return TV_ERR_BAD_ARGUMENT;
+    tv::SnapshotInfo info;
+    const std::string why = tv::snapshot_parse(bytes, len, info);
+    if (!why.empty()) { g_last_error = why; return TV_ERR_BAD_IMAGE; }
+    const size_t nl = size_t(1) << info.bits;
+    if (boundaries) std::memcpy(boundaries, bytes + info.boundaries_at, (nl - 1) * 4);
+    if (centroids) std::memcpy(centroids, bytes + info.centroids_at, nl * 4);
+    if (shift) std::memcpy(shift, bytes + info.shift_at, info.n_calib * 4);
+    if (scale) std::memcpy(scale, bytes + info.scale_at, info.n_calib * 4);
+    if (seq || scales || ids) {
+        const size_t nb = (info.n + 31) / 32;
+        std::vector<uint8_t> seq_tmp;
+        std::vector<float> sc_tmp;
+        if (!seq) { seq_tmp.resize(nb * info.row_bytes * 32); seq = seq_tmp.data(); }
+        if (!scales) { sc_tmp.resize(nb * 32); scales = sc_tmp.data(); }
+        tv::snapshot_extract(bytes, info, seq, scales, ids);
+    }
+    return TV_OK;
+}
+
+int tv_index_to_bytes(const tv_index *ix, const uint64_t *ids, int format, uint8_t *out, size_t cap, size_t *len) {
+    if (!ix || !len || (format != 6 && format != 7)) return TV_ERR_BAD_ARGUMENT;
+    const int kind = ids ? 1 : 0;
+    const size_t n = ix->n, n_calib = ix->tq_shift.size();
+    *len = tv::snapshot_len(format, ix->geo.dim, ix->geo.bits, kind, n_calib, n);
+    if (!out) return TV_OK;
+    if (cap < *len) return TV_ERR_BAD_ARGUMENT;
+    const size_t nb = (n + 31) / 32;
+    std::vector<uint8_t> seq(nb * size_t(ix->geo.G) * 32);
+    std::vector<float> scales(n);
+    int rc = tv_index_download_seq(ix, seq.data(), scales.data());
+    if (rc != TV_OK) return rc;
+    const tv::SnapshotParts s{kind, ix->geo.dim, ix->geo.bits, ix->cb.boundaries.data(), ix->cb.centroids.data(),
+                              n_calib, ix->tq_shift.data(), ix->tq_scale.data(), seq.data(), n, scales.data(), ids};
+    tv::snapshot_compose(format, s, out);
+    return TV_OK;
+}
+
+int tv_index_from_bytes(const uint8_t *bytes, size_t len, int device, tv_index **out, uint64_t *ids_out) {
+    if (!bytes || !out) return TV_ERR_BAD_ARGUMENT;
+    *out = nullptr;
+    tv::SnapshotInfo info;
+    const std::string why = tv::snapshot_parse(bytes, len, info);
+    if (!why.empty()) { g_last_error = why; return TV_ERR_BAD_IMAGE; }
+    tv_index *ix = nullptr;
+    int rc = tv_index_create(info.dim, info.bits, device, &ix);
+    if (rc != TV_OK) return rc;
+    const size_t nl = size_t(1) << info.bits;
+    std::vector<float> cen(nl), sh(info.n_calib), sc(info.n_calib);
+    std::memcpy(cen.data(), bytes + info.centroids_at, nl * 4);
+    std::memcpy(sh.data(), bytes + info.shift_at, info.n_calib * 4);
+    std::memcpy(sc.data(), bytes + info.scale_at, info.n_calib * 4);
+    rc = tv_index_set_tables(ix, nullptr, nullptr, cen.data());
+    if (rc == TV_OK && info.n_calib) rc = tv_index_set_calibration(ix, sh.data(), sc.data());
+    if (rc == TV_OK && info.n) {
+        const size_t nb = (info.n + 31) / 32;
+        std::vector<uint8_t> seq(nb * info.row_bytes * 32);
+        std::vector<float> scales(nb * 32);
+        tv::snapshot_extract(bytes, info, seq.data(), scales.data(), ids_out);
+        rc = tv_index_upload_seq(ix, seq.data(), info.n, scales.data());
+    }
+    if (rc != TV_OK) { tv_index_destroy(ix); return rc; }
+    *out = ix;
     return TV_OK;
 }
 

@@ -10,9 +10,15 @@ its C ABI: encode on add, lane moves on swap_remove, and the whole search.  The
 id <-> slot tables stay on the host, as in the reference.  There is no CPU
 search here: without the built library every method raises ImportError.
 
-Not mirrored (outside the search path): write/load/sync, calibrate (the TQ+
-fit; a fitted pair can be handed over with `set_calibration`), pickling.
+Snapshots: `to_bytes` / `from_bytes` / `write` / `load` produce and read the
+reference's image bytes (turbovec/src/io_v7.rs; lib.rs:2167 to_bytes, id_map.rs:971)
+through tv_index_to_bytes / tv_index_from_bytes.
+
+Not mirrored (outside the search path): sync (the incremental container),
+calibrate (the TQ+ fit; a fitted pair can be handed over with
+`set_calibration`), pickling.
 """
+import os
 import threading
 
 import numpy as np
@@ -95,6 +101,30 @@ class TurboQuantIndex:
         with self._lock:
             self._ix.set_calibration(shift, scale)
 
+    # -- snapshots ---------------------------------------------------------
+    def to_bytes(self):
+        with self._lock:
+            return self._ix.to_bytes()
+
+    @classmethod
+    def from_bytes(cls, data, device=0):
+        return cls._adopt(*_load_image(data, device, want_kind=0))
+
+    @classmethod
+    def _adopt(cls, native, _ids):
+        self = cls.__new__(cls)
+        self._ix = native
+        self._lock = threading.RLock()
+        return self
+
+    def write(self, path):
+        _write_atomically(path, self.to_bytes())
+
+    @classmethod
+    def load(cls, path, device=0):
+        with open(path, "rb") as f:
+            return cls.from_bytes(f.read(), device)
+
     # -- mutation ----------------------------------------------------------
     def add(self, vectors):
         v = _f32_2d("vectors", vectors)
@@ -153,6 +183,31 @@ class TurboQuantIndex:
         return self._ix.search(q, k_lib, mask_words=words)
 
 
+def _load_image(data, device, want_kind):
+    """Corrupt or foreign bytes surface as a plain OSError, as the reference's loaders do."""
+    try:
+        info = T.snapshot_info(data)
+        if info[1] != want_kind:
+            raise OSError("image holds %s index" % ("an id-map" if info[1] == 1 else "a slot-addressed"))
+        return T.NativeIndex.from_bytes(data, device)
+    except T.TurbovecHipError as e:
+        raise OSError(str(e)) from None
+
+
+def _write_atomically(path, data):
+    """Temp sibling + rename: the destination never holds a torn image."""
+    path = os.fspath(path)
+    d = os.path.dirname(path) or "."
+    if not os.path.isdir(d):
+        raise FileNotFoundError(f"cannot write {path!r}: directory {d!r} does not exist")
+    tmp = f"{path}.tmp.{os.getpid()}"
+    with open(tmp, "wb") as f:
+        f.write(data)
+        f.flush()
+        os.fsync(f.fileno())
+    os.replace(tmp, path)
+
+
 class IdMapIndex:
     """Index addressed by external uint64 ids; `search` returns (scores, ids uint64)."""
 
@@ -174,6 +229,29 @@ class IdMapIndex:
 
     def prepare(self):
         return None
+
+    def to_bytes(self):
+        with self._inner._lock:
+            return self._inner._ix.to_bytes(ids=np.asarray(self._slot_to_id, np.uint64))
+
+    @classmethod
+    def from_bytes(cls, data, device=0):
+        native, ids = _load_image(data, device, want_kind=1)
+        self = cls.__new__(cls)
+        self._inner = TurboQuantIndex._adopt(native, None)
+        self._slot_to_id = ids.tolist()
+        self._id_to_slot = {x: i for i, x in enumerate(self._slot_to_id)}
+        if len(self._id_to_slot) != len(self._slot_to_id):
+            raise OSError("image holds duplicate ids")
+        return self
+
+    def write(self, path):
+        _write_atomically(path, self.to_bytes())
+
+    @classmethod
+    def load(cls, path, device=0):
+        with open(path, "rb") as f:
+            return cls.from_bytes(f.read(), device)
 
     def contains(self, id):
         try:
