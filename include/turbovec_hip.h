@@ -96,6 +96,15 @@ int tv_index_append_rows(tv_index *ix, const uint8_t *rows, const float *scales,
  * :900-932).  Values must be finite with |x| < 1e16 (encode.rs:76-83):
  * TV_ERR_INVALID_QUERY_VALUE otherwise, and nothing is added. */
 int tv_index_add(tv_index *ix, const float *vectors, size_t n_new);
+/* Fit the TQ+ per-coordinate pair from n >= 2 sample rows and commit it
+ * (TurboQuantIndex::calibrate, lib.rs:2599; fit encode.rs:737-857): the sample is
+ * normalised and rotated on the device, the order statistics are taken on the
+ * host.  Only on an empty index: re-encoding stored rows under a new pair
+ * (lib.rs:2599-2835) is not built.  The fitted pair equals the reference's bit
+ * for bit. */
+int tv_index_calibrate(tv_index *ix, const float *sample, size_t n);
+/* The committed pair: *n_calib is 0 (uncalibrated) or dim; shift/scale may be NULL. */
+int tv_index_get_calibration(const tv_index *ix, float *shift, float *scale, size_t *n_calib);
 /* Same, rows already in device memory (not validated: the caller checked them). */
 int tv_index_add_dev(tv_index *ix, const float *d_vectors, size_t n_new);
 /* lib.rs:2864-3028: move the last vector into slot idx, zero the vacated lane. */

@@ -28,9 +28,12 @@ def test_fingerprint_cells_encoded_on_device(T, oracle, row):
     v = O.lcg_vectors(2000, dim, fingerprint_seed(dim, bits))
     rot = O.Rotation(dim)
     _b, c = O.codebook(bits, dim)
-    sh, sc = O.fit_calibration(rot, v, c)          # the fixture calibrates before it adds
     ix = T.NativeIndex(dim, bits)
-    ix.set_calibration(sh, sc)
+    ix.calibrate(v)                                # the fixture calibrates before it adds
+    sh, sc = ix.calibration()
+    assert O.fnv1a(np.concatenate([sh, sc])) == _wcal          # the fit itself: rotated on the device, ranked on the host
+    osh, osc = O.fit_calibration(rot, v, c)
+    assert bits_equal(sh, osh) and bits_equal(sc, osc)
     ix.add(v)
     assert len(ix) == 2000
     seq, scales = ix.download_seq()

@@ -258,3 +258,23 @@ def test_allowlist_semantics(api):
     assert idx.remove(int(ids[1]))
     s, g = idx.search(q, 100, allowlist=ids[[5, 9, 399]])
     assert s.shape == (5, 3) and set(g[0].tolist()) == set(ids[[5, 9, 399]].tolist())
+
+
+def test_calibrate_before_add(api):
+    v = unit_vectors(600, dim=256, seed=21) * np.linspace(0.2, 3.0, 256, dtype=np.float32)   # anisotropic
+    v /= np.linalg.norm(v, axis=1, keepdims=True)
+    idx = api.TurboQuantIndex(256, 4)
+    assert idx.calibration_state == "uncalibrated"
+    idx.calibrate(v)
+    assert idx.calibration_state == "calibrated"
+    idx.add(v)
+    _, i = idx.search(v[:100], 1)
+    assert (i[:, 0] == np.arange(100)).mean() >= 0.99
+    again = api.TurboQuantIndex.from_bytes(idx.to_bytes())
+    assert again.calibration_state == "calibrated" and again.to_bytes() == idx.to_bytes()
+    with pytest.raises(NotImplementedError):
+        idx.calibrate(v)
+    with pytest.raises(ValueError):
+        api.TurboQuantIndex(256, 4).calibrate(v[:1])
+    with pytest.raises(TypeError):
+        api.TurboQuantIndex(256, 4).calibrate(v.astype(np.float64))

@@ -27,7 +27,7 @@ SCORE_AUTO, SCORE_L_CLASSIC, SCORE_L_U32, SCORE_P = 0, 2, 3, 4
 EXPORTS = [
     "tv_status_string", "tv_last_error", "tv_index_create", "tv_index_destroy", "tv_index_set_tables",
     "tv_index_set_calibration", "tv_index_set_score_mode", "tv_index_get_tables", "tv_index_upload_seq",
-    "tv_index_upload_seq_dev", "tv_index_append_rows", "tv_index_add", "tv_index_add_dev", "tv_index_swap_remove", "tv_index_download_seq", "tv_index_len", "tv_index_dim",
+    "tv_index_upload_seq_dev", "tv_index_append_rows", "tv_index_add", "tv_index_add_dev", "tv_index_calibrate", "tv_index_get_calibration", "tv_index_swap_remove", "tv_index_download_seq", "tv_index_len", "tv_index_dim",
     "tv_index_bits", "tv_validate_queries", "tv_pack_mask", "tv_search", "tv_search_dev", "tv_debug_scan",
     "tv_debug_prepare", "tv_last_scan_ms", "tv_index_device_ptrs", "tv_host_rotation_tables", "tv_host_codebook",
     "tv_debug_stream_probe", "tv_debug_set_path", "tv_debug_overflow_redos",
@@ -68,6 +68,8 @@ def lib():
     L.tv_index_upload_seq_dev.argtypes = [vp, vp, sz, vp]
     L.tv_index_append_rows.argtypes = [vp, vp, vp, sz]
     L.tv_index_add.argtypes = [vp, vp, sz]
+    L.tv_index_calibrate.argtypes = [vp, vp, sz]
+    L.tv_index_get_calibration.argtypes = [vp, vp, vp, C.POINTER(sz)]
     L.tv_host_snapshot_len.restype = sz
     L.tv_host_snapshot_len.argtypes = [i32, i32, i32, i32, sz, sz]
     L.tv_host_snapshot_compose.argtypes = [i32, i32, i32, i32, vp, vp, sz, vp, vp, vp, sz, vp, vp, vp]
@@ -177,6 +179,20 @@ class NativeIndex:
         """Encode raw float32 rows on the device and append them (tv_index_add)."""
         v = np.ascontiguousarray(vectors, np.float32).reshape(-1, self.dim)
         check(lib().tv_index_add(self.h, ptr(v), len(v)))
+
+    def calibrate(self, sample):
+        """Fit and commit the TQ+ pair from sample rows (tv_index_calibrate); empty index only."""
+        v = np.ascontiguousarray(sample, np.float32).reshape(-1, self.dim)
+        check(lib().tv_index_calibrate(self.h, ptr(v), len(v)))
+
+    def calibration(self):
+        n = C.c_size_t(0)
+        check(lib().tv_index_get_calibration(self.h, None, None, C.byref(n)))
+        if n.value == 0:
+            return None
+        sh, sc = np.zeros(n.value, np.float32), np.zeros(n.value, np.float32)
+        check(lib().tv_index_get_calibration(self.h, ptr(sh), ptr(sc), C.byref(n)))
+        return sh, sc
 
     def add_dev(self, d_vectors_ptr, n):
         check(lib().tv_index_add_dev(self.h, d_vectors_ptr, n))

@@ -1,5 +1,8 @@
 #include "host_tables.h"
 
+#include <algorithm>
+#include <cstring>
+
 #include <array>
 #include <cfloat>
 #include <cmath>
@@ -194,6 +197,39 @@ Codebook make_codebook(int bits, int dim) {
     std::lock_guard<std::mutex> lock(mu);
     memo[{bits, dim}] = cb;
     return cb;
+}
+
+void fit_tqplus(const float *rotated, size_t n, int dim, const std::vector<float> &centroids,
+                float *shift, float *scale) {
+    float c_outer = 0.0f;
+    for (float c : centroids) c_outer = std::fmax(c_outer, std::fabs(c));
+    const double shape = (double(dim) - 1.0) / 2.0;
+    const double p_hi = incomplete_beta_sym(shape, (double(c_outer) + 1.0) / 2.0);   // encode.rs:364-369
+    const double p_lo = 1.0 - p_hi;
+    const float qc_lo = -c_outer, qc_span = c_outer - qc_lo;
+    size_t lo_idx = size_t(double(n) * p_lo);
+    size_t hi_idx = size_t(double(n) * p_hi);
+    if (hi_idx > n - 1) hi_idx = n - 1;
+    if (hi_idx < lo_idx + 1) hi_idx = lo_idx + 1;
+    // total order of encode.rs:183-186: sign-magnitude bits mapped to unsigned keys
+    auto key = [](float x) { uint32_t b; std::memcpy(&b, &x, 4); return b ^ (uint32_t(int32_t(b) >> 31) | 0x80000000u); };
+    auto unkey = [](uint32_t k) { const uint32_t b = k ^ ((k & 0x80000000u) ? 0x80000000u : 0xFFFFFFFFu); float x; std::memcpy(&x, &b, 4); return x; };
+    std::vector<uint32_t> col(n);
+    for (int d = 0; d < dim; ++d) {
+        shift[d] = 0.0f;
+        scale[d] = 1.0f;
+        if (n < 2 || hi_idx >= n) continue;
+        for (size_t i = 0; i < n; ++i) col[i] = key(rotated[i * size_t(dim) + d]);
+        std::nth_element(col.begin(), col.begin() + lo_idx, col.end());
+        const float qe_lo = unkey(col[lo_idx]);
+        std::nth_element(col.begin() + lo_idx + 1, col.begin() + hi_idx, col.end());   // hi_idx > lo_idx
+        const float qe_hi = unkey(col[hi_idx]);
+        const float qe_span = qe_hi - qe_lo;
+        if (qe_span > 1e-6f) {
+            scale[d] = qc_span / qe_span;
+            shift[d] = qc_lo / scale[d] - qe_lo;
+        }
+    }
 }
 
 }  // namespace tv

@@ -26,4 +26,11 @@ struct Codebook {
 // turbovec/src/codebook.rs:69-167 (lloyd_max, 200 iterations, tol 1e-12).
 Codebook make_codebook(int bits, int dim);
 
+// turbovec/src/encode.rs:737-857 (compute_tqplus_calibration) given the rotated unit rows
+// (n * dim floats, row-major): per coordinate, the order statistics at the tail
+// probabilities of the outer centroid under Beta((dim-1)/2, (dim-1)/2) are mapped onto
+// +-outer centroid.  shift and scale receive dim floats each.
+void fit_tqplus(const float *rotated, size_t n, int dim, const std::vector<float> &centroids,
+                float *shift, float *scale);
+
 }  // namespace tv

@@ -650,7 +650,7 @@ static int add_device_rows(tv_index *ix, const float *d_vectors, size_t n_new) {
         TV_HIP(tv::launch_encode(d_vectors + r0 * size_t(g.dim), nr, ix->n + r0, ix->d_signs, ix->d_perms,
                                  cal ? ix->d_tq_shift : nullptr, cal ? ix->d_tq_scale : nullptr,
                                  ix->cb.centroids.data(), ix->cb.boundaries.data(), g, ix->rot.block,
-                                 ix->rot.inv_sqrt_block, ix->d_codes, ix->d_scales, ix->stream));
+                                 ix->rot.inv_sqrt_block, ix->d_codes, ix->d_scales, nullptr, ix->stream));
     }
     TV_HIP(hipStreamSynchronize(ix->stream));
     ix->n += n_new;
@@ -692,6 +692,54 @@ int tv_index_add(tv_index *ix, const float *vectors, size_t n_new) {
         rc = add_device_rows(ix, static_cast<const float *>(ix->ws), nr);
         if (rc != TV_OK) return rc;
     }
+    return TV_OK;
+}
+
+// TurboQuantIndex::calibrate (lib.rs:2599) on an empty index: rotate the normalised sample on
+// the device (encode.rs:406-458), fit on the host (encode.rs:737-857), commit the pair.
+int tv_index_calibrate(tv_index *ix, const float *sample, size_t n) {
+    if (!ix || !sample) return TV_ERR_BAD_ARGUMENT;
+    if (n < 2) { g_last_error = "calibration needs at least 2 rows"; return TV_ERR_BAD_ARGUMENT; }   // encode.rs:395
+    const size_t dim = size_t(ix->geo.dim);
+    size_t bad = 0;
+    int rc = tv_validate_queries(sample, n * dim, ix->geo.dim, &bad);
+    if (rc != TV_OK) {
+        g_last_error = "sample row " + std::to_string(bad / dim) + " holds a non-finite or too large value";
+        return rc;
+    }
+    std::vector<float> rotated(n * dim);
+    {
+        std::lock_guard<std::mutex> lock(ix->mu);
+        if (ix->n != 0) {
+            g_last_error = "calibrate on a populated index (re-encoding stored rows) is not supported";
+            return TV_ERR_BAD_ARGUMENT;
+        }
+        TV_HIP(hipSetDevice(ix->device));
+        const size_t slice = std::max<size_t>(1, (size_t(128) << 20) / (dim * sizeof(float)));
+        rc = ensure_workspace(ix, 2 * std::min(n, slice) * dim * sizeof(float) + 512);
+        if (rc != TV_OK) return rc;
+        float *d_in = static_cast<float *>(ix->ws);
+        float *d_out = d_in + std::min(n, slice) * dim;
+        for (size_t r0 = 0; r0 < n; r0 += slice) {
+            const size_t nr = std::min(slice, n - r0);
+            TV_HIP(hipMemcpyAsync(d_in, sample + r0 * dim, nr * dim * sizeof(float), hipMemcpyHostToDevice, ix->stream));
+            TV_HIP(tv::launch_encode(d_in, nr, 0, ix->d_signs, ix->d_perms, nullptr, nullptr, ix->cb.centroids.data(),
+                                     ix->cb.boundaries.data(), ix->geo, ix->rot.block, ix->rot.inv_sqrt_block,
+                                     nullptr, nullptr, d_out, ix->stream));
+            TV_HIP(hipMemcpyAsync(rotated.data() + r0 * dim, d_out, nr * dim * sizeof(float), hipMemcpyDeviceToHost, ix->stream));
+            TV_HIP(hipStreamSynchronize(ix->stream));
+        }
+    }
+    std::vector<float> shift(dim), scale(dim);
+    tv::fit_tqplus(rotated.data(), n, ix->geo.dim, ix->cb.centroids, shift.data(), scale.data());
+    return tv_index_set_calibration(ix, shift.data(), scale.data());
+}
+
+int tv_index_get_calibration(const tv_index *ix, float *shift, float *scale, size_t *n_calib) {
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    if (n_calib) *n_calib = ix->tq_shift.size();
+    if (shift && !ix->tq_shift.empty()) std::memcpy(shift, ix->tq_shift.data(), ix->tq_shift.size() * sizeof(float));
+    if (scale && !ix->tq_scale.empty()) std::memcpy(scale, ix->tq_scale.data(), ix->tq_scale.size() * sizeof(float));
     return TV_OK;
 }
 

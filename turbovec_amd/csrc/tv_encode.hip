@@ -26,6 +26,7 @@ struct EncodeArgs {
     float bnd[16];
     int dim, bits, G, nch, block;
     float inv_sqrt_block;
+    float *rot_out;           // when set: write the rotated unit rows here and stop (TQ+ fit input)
     uint8_t *nat;             // codes in the device layout
     float *scales;
     size_t old_n, n_new;
@@ -84,6 +85,11 @@ __global__ __launch_bounds__(256) void k_encode(EncodeArgs a) {
     wht_lds(A, dim, a.block, t);
     for (int i = t; i < dim; i += 256) B[i] = A[i] * a.inv_sqrt_block;   // B = rotated unit row
     __syncthreads();
+    if (a.rot_out != nullptr) {
+        float *dst = a.rot_out + row * size_t(dim);
+        for (int i = t; i < dim; i += 256) dst[i] = B[i];
+        return;
+    }
 
     // encode.rs:600-640: code = number of boundaries below the calibrated value
     uint8_t *codes = reinterpret_cast<uint8_t *>(A);
@@ -131,7 +137,8 @@ __global__ __launch_bounds__(256) void k_encode(EncodeArgs a) {
 hipError_t launch_encode(const float *d_vecs, size_t n_new, size_t old_n, const float *d_signs,
                          const uint32_t *d_perms, const float *d_shift, const float *d_scale,
                          const float *centroids, const float *boundaries, const Geometry &g, int block,
-                         float inv_sqrt_block, uint8_t *d_native, float *d_scales, hipStream_t s) {
+                         float inv_sqrt_block, uint8_t *d_native, float *d_scales, float *d_rot_out,
+                         hipStream_t s) {
     if (n_new == 0) return hipSuccess;
     EncodeArgs a;
     a.vecs = d_vecs; a.signs = d_signs; a.perms = d_perms; a.shift = d_shift; a.scale = d_scale;
@@ -140,6 +147,7 @@ hipError_t launch_encode(const float *d_vecs, size_t n_new, size_t old_n, const 
     a.dim = g.dim; a.bits = g.bits; a.G = g.G; a.nch = g.nch; a.block = block;
     a.inv_sqrt_block = inv_sqrt_block;
     a.nat = d_native; a.scales = d_scales; a.old_n = old_n; a.n_new = n_new;
+    a.rot_out = d_rot_out;
     const size_t lds = size_t(2) * g.dim * sizeof(float);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_encode),

@@ -76,7 +76,8 @@ hipError_t launch_append_rows(const uint8_t *d_rows, uint8_t *d_native, const Ge
 hipError_t launch_encode(const float *d_vecs, size_t n_new, size_t old_n, const float *d_signs,
                          const uint32_t *d_perms, const float *d_shift, const float *d_scale,
                          const float *centroids, const float *boundaries, const Geometry &g, int block,
-                         float inv_sqrt_block, uint8_t *d_native, float *d_scales, hipStream_t s);
+                         float inv_sqrt_block, uint8_t *d_native, float *d_scales, float *d_rot_out,
+                         hipStream_t s);
 hipError_t launch_move_lane(uint8_t *d_native, float *d_scales, const Geometry &g, size_t src, size_t dst,
                             hipStream_t s);
 

@@ -15,8 +15,7 @@ reference's image bytes (turbovec/src/io_v7.rs; lib.rs:2167 to_bytes, id_map.rs:
 through tv_index_to_bytes / tv_index_from_bytes.
 
 Not mirrored (outside the search path): sync (the incremental container),
-calibrate (the TQ+ fit; a fitted pair can be handed over with
-`set_calibration`), pickling.
+calibrate on a populated index (re-encoding stored rows), pickling.
 """
 import os
 import threading
@@ -95,6 +94,23 @@ class TurboQuantIndex:
     def prepare(self):
         """Idempotent; the device copy of the index is always search-ready."""
         return None
+
+    def calibrate(self, sample):
+        """Fit the TQ+ pair from `sample` and commit it (lib.rs:2599); before the first add only."""
+        v = _f32_2d("sample", sample)
+        if v.shape[1] != self.dim:
+            raise ValueError(f"sample dim {v.shape[1]} does not match index dim {self.dim}")
+        if len(v) < 2:
+            raise ValueError("calibration needs at least 2 rows")
+        _check_values("sample", v, "sample row")
+        with self._lock:
+            if len(self._ix):
+                raise NotImplementedError("calibrate on a populated index (re-encoding stored rows) is not built")
+            self._ix.calibrate(v)
+
+    @property
+    def calibration_state(self):
+        return "uncalibrated" if self._ix.calibration() is None else "calibrated"
 
     def set_calibration(self, shift, scale):
         """Hand over a fitted TQ+ pair (turbovec/src/lib.rs:2599); affects later adds and searches."""
