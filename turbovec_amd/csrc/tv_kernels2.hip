@@ -22,6 +22,10 @@ namespace tv {
 // waves per SIMD, which is what hides the LDS and HBM latencies.
 // ===========================================================================
 
+typedef uint32_t lut_u32x2 __attribute__((ext_vector_type(2)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
 // base + byte E of packed, in one instruction (sub-dword operand select).
 template <int E>
 __device__ __forceinline__ uint32_t add_byte(uint32_t base, uint32_t packed) {
@@ -33,6 +37,22 @@ __device__ __forceinline__ uint32_t add_byte(uint32_t base, uint32_t packed) {
     return r;
 }
 
+// The m-th A operand (16 bytes) out of a lane's 16 looked-up table words.
+template <int QL, typename W>
+__device__ __forceinline__ v4i lut_a_operand(const W (&w)[16], int m);
+template <>
+__device__ __forceinline__ v4i lut_a_operand<4, uint32_t>(const uint32_t (&w)[16], int m) {
+    return v4i{int(w[4 * m]), int(w[4 * m + 1]), int(w[4 * m + 2]), int(w[4 * m + 3])};
+}
+template <>
+__device__ __forceinline__ v4i lut_a_operand<8, lut_u32x2>(const lut_u32x2 (&w)[16], int m) {
+    return v4i{int(w[2 * m].x), int(w[2 * m].y), int(w[2 * m + 1].x), int(w[2 * m + 1].y)};
+}
+template <>
+__device__ __forceinline__ v4i lut_a_operand<1, uint8_t>(const uint8_t (&)[16], int) { return v4i{0, 0, 0, 0}; }
+template <>
+__device__ __forceinline__ v4i lut_a_operand<2, uint16_t>(const uint16_t (&)[16], int) { return v4i{0, 0, 0, 0}; }
+
 template <int V> struct IntC { static constexpr int value = V; };
 template <typename F>
 __device__ __forceinline__ void static_for4(F &&f) { f(IntC<0>{}); f(IntC<1>{}); f(IntC<2>{}); f(IntC<3>{}); }
@@ -41,7 +61,6 @@ template <int QL> struct LutWord;
 template <> struct LutWord<1> { typedef uint8_t type; };
 template <> struct LutWord<2> { typedef uint16_t type; };
 template <> struct LutWord<4> { typedef uint32_t type; };
-typedef uint32_t lut_u32x2 __attribute__((ext_vector_type(2)));
 template <> struct LutWord<8> { typedef lut_u32x2 type; };
 
 // acc[q] += byte q of (vh + vl), bytewise sums never carrying (entries <= 127).
@@ -110,6 +129,20 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
     uint32_t *scnt = reinterpret_cast<uint32_t *>(stau);  // append mode: candidates per query of this workgroup
     if (APPEND && tid < kQTile) scnt[tid] = 0u;
     __syncthreads();
+    // With whole-dword table words (4 or 8 queries) the per-query sums are taken by the matrix
+    // unit: a lane's looked-up words are an A operand as they are (row = its vector, 16 bytes =
+    // a few groups x QL queries), and B[k][n] = 1 where byte k belongs to query n adds them up
+    // per query in 32-bit integers while the vector ALU moves on to the next addresses.
+    constexpr bool MF = LUT_LDS && (QL == 4 || QL == 8);
+    v4i bsel = {0, 0, 0, 0};
+    {
+        const int n = threadIdx.x & 31;
+        if (QL == 4) { const int w = n < 4 ? int(1u << (8 * n)) : 0; bsel = v4i{w, w, w, w}; }
+        if (QL == 8) {
+            const int w0 = n < 4 ? int(1u << (8 * n)) : 0, w1 = (n >= 4 && n < 8) ? int(1u << (8 * (n - 4))) : 0;
+            bsel = v4i{w0, w1, w0, w1};
+        }
+    }
     const word_t *lut = LUT_LDS ? reinterpret_cast<const word_t *>(smem) : reinterpret_cast<const word_t *>(a.tables);
     // the tables' address inside LDS as a plain number: entry addresses are then formed with integer
     // adds and dereferenced as LDS pointers, with the per-byte row offsets riding in the read's offset field
@@ -167,6 +200,8 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
         uint32_t acc[QL];
 #pragma unroll
         for (int qq = 0; qq < QL; ++qq) acc[qq] = 0;
+        v16i macc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        word_t wh[16], wl[16];
         for (int c0 = 0; c0 < nch; c0 += U) {
             uint4 cur[U];
 #pragma unroll
@@ -203,13 +238,39 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
                             vh = *reinterpret_cast<const word_t *>(gbase + add_byte<e>(row_off, phi) + j * 32 * QL);
                             vl = *reinterpret_cast<const word_t *>(gbase + add_byte<e>(row_off, plo) + (j * 32 + 16) * QL);
                         }
-                        LutAcc<QL>::add(acc, vh, vl);
+                        if (MF) { wh[j] = vh; wl[j] = vl; }
+                        else LutAcc<QL>::add(acc, vh, vl);
                     });
                 }
+                if (MF) {
+                    // 16 bytes of a lane = WPA groups x QL queries; the one-hot B sums them per query
+                    constexpr int WPA = 16 / QL;   // words per A operand
+#pragma unroll
+                    for (int m = 0; m < 16 / WPA; ++m) {
+                        macc = __builtin_amdgcn_mfma_i32_32x32x32_i8(lut_a_operand<QL>(wh, m), bsel, macc, 0, 0, 0);
+                        macc = __builtin_amdgcn_mfma_i32_32x32x32_i8(lut_a_operand<QL>(wl, m), bsel, macc, 0, 0, 0);
+                    }
+                }
                 if ((c & 7) == 7 || c == nch - 1) {  // end of a 256-group batch (search.rs:529-531)
+                    if (MF) {
+                        // query q's sums sit in the lanes of output column q: hand them to the lanes
+                        // of their vectors through the wave's scratch rows
+                        int *xch = reinterpret_cast<int *>(my_sct);
+                        if (vi < QL) {
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) xch[vi * 32 + 8 * (r >> 2) + 4 * h + (r & 3)] = macc[r];
+                        }
+                        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+                        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                        for (int qq = 0; qq < QL; ++qq) acc[qq] = uint32_t(xch[qq * 32 + vi]);
+                        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+                        __builtin_amdgcn_wave_barrier();
+                        macc = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    }
 #pragma unroll
                     for (int qq = 0; qq < QL; ++qq) {
-                        const uint32_t part = acc[qq] + uint32_t(__shfl_xor(int(acc[qq]), 32));
+                        const uint32_t part = MF ? acc[qq] : acc[qq] + uint32_t(__shfl_xor(int(acc[qq]), 32));
                         acc[qq] = 0;
                         total[qq] += part;
                         fa[qq] = fmaf(qs[qq], float(part), fa[qq]);  // search.rs:577-580
