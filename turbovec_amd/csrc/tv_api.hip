@@ -137,7 +137,7 @@ int prepare_queries(tv_index *ix, Arena &ar, const float *d_q, size_t nq, Prepar
         TV_HIP(tv::launch_calibrate(d_rot, d_cal, d_bias_corr, ix->d_tq_shift, ix->d_tq_scale, g.dim, nq,
                                     ix->stream));
     } else {
-        TV_HIP(tv::launch_fill_i32(reinterpret_cast<int *>(d_bias_corr), 0, nq_pad, ix->stream));
+        d_bias_corr = nullptr;   // uncalibrated: the table builders add +0.0f themselves (search.rs:3176-3185)
     }
     out.d_qrot = d_cal;
     out.d_qscale = ar.take<float>(nq_pad);
@@ -177,6 +177,8 @@ void fill_scan_args(const tv_index *ix, tv::ScanArgs &a) {
 }
 
 constexpr size_t kChunkQueries = 1024;
+// a chunk's floors are laid out tile by tile, kQTile slots per tile, and a tile may hold one query
+constexpr size_t kTauOpenInts = kChunkQueries * tv::kQTile;
 constexpr int kMaxTimedTiles = int(kChunkQueries / tv::kQTile);
 
 struct EventPool {
@@ -283,24 +285,24 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
 }
 
 // Sampling plan of a search: block strides of the successive append-mode scans,
-// the last one being 1 (the full scan).  Sizes shrink from the full index by
-// the factor target/k_floor per level until a level is small enough for all of
-// its slots to be appended; each later level, filtered by the floor of the one
-// before, then appends about `target` candidates per query, and the sampling
-// levels together read only about k_floor/target of the index.
+// the last one being 1 (the full scan).  The first level reads about `first`
+// slots and, having no floor yet, appends all of them (one short sort); level
+// sizes then grow geometrically to the full index, by a factor chosen so that
+// a level filtered by the floor of the one before appends at most about 2048
+// candidates per query (the floor is the k_floor-th best of the level before,
+// so a level `ratio` times larger keeps about ratio * k_floor).  The sampling
+// levels together read about 1/ratio of the index.
 std::vector<uint32_t> sampling_steps(size_t n_blocks, size_t k_floor) {
     const double n_slots = double(n_blocks * tv::kVecBlock);
-    const double target = double(std::max<size_t>(1024, 4 * k_floor));
-    const double ratio = target / double(k_floor);
+    const double first = double(std::max<size_t>(1024, 8 * k_floor));
     std::vector<uint32_t> steps;
-    std::vector<double> sizes;
-    for (double sample = n_slots / ratio; ; sample /= ratio) {
-        sizes.push_back(sample);
-        if (sample <= target) break;
-    }
-    if (n_slots > target) {
-        for (size_t i = sizes.size(); i-- > 0;) {
-            const size_t sample_blocks = std::max<size_t>(1, size_t(sizes[i]) / tv::kVecBlock);
+    if (n_slots > 2.0 * first) {
+        const double max_ratio = std::max(4.0, 2048.0 / double(k_floor));
+        const int levels = std::max(1, int(std::ceil(std::log(n_slots / first) / std::log(max_ratio))));
+        const double ratio = std::pow(n_slots / first, 1.0 / double(levels));
+        double sample = first;
+        for (int lv = 0; lv < levels; ++lv, sample *= ratio) {
+            const size_t sample_blocks = std::max<size_t>(1, size_t(sample) / tv::kVecBlock);
             const size_t step = n_blocks / sample_blocks;
             if (step > 1 && (steps.empty() || step < steps.back())) steps.push_back(uint32_t(step));
         }
@@ -365,8 +367,8 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
         uint64_t *d_cand = ar.take<uint64_t>(cq_pad * seg_stride * tv::kSegCap);
         uint32_t *d_cnt = ar.take<uint32_t>(cq_pad * seg_stride);
         uint32_t *d_over = ar.take<uint32_t>(cq_pad);
-        TV_HIP(tv::launch_fill_i32(d_tau, int(0x807fffffu) /* order key of -inf */, n_tiles * tv::kQTile, ix->stream));
-        TV_HIP(tv::launch_fill_i32(reinterpret_cast<int *>(d_over), 0, cq_pad, ix->stream));
+        // no per-search clears: the first level reads the index's standing array of open floors,
+        // every later one the floors k_final wrote, and k_final writes every overflow flag
 
         const int nt_batched = (mode_p && cq > size_t(tv::kQTile) && !ix->no_batched) ? tv::batched_tiles(g.nch) : 0;
         const int bgrid = tv::batched_grid_blocks(ix->device, g.nch);
@@ -388,7 +390,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
                 a.qbias = pq.d_qbias + t * tile_q;
                 a.nq_tile = int(std::min<size_t>(tile_q * tiles_per_launch, cq - t * tile_q));
                 a.k = 1;
-                a.gtau = d_tau + t * tv::kQTile;
+                a.gtau = (lv == 0 ? ix->d_tau_open : d_tau) + t * tv::kQTile;
                 a.b_step = steps[lv];
                 a.cand = d_cand + t * tile_q * seg_stride * tv::kSegCap;
                 a.cand_cnt = d_cnt + t * tile_q * seg_stride;
@@ -486,7 +488,14 @@ int tv_index_create(int dim, int bits, int device, tv_index **out) {
             hipMalloc(reinterpret_cast<void **>(&ix->d_perms), 2 * size_t(dim) * sizeof(uint32_t)) != hipSuccess ||
             hipMalloc(reinterpret_cast<void **>(&ix->d_centroids), 16 * sizeof(float)) != hipSuccess ||
             hipMalloc(reinterpret_cast<void **>(&ix->d_tq_shift), size_t(dim) * sizeof(float)) != hipSuccess ||
-            hipMalloc(reinterpret_cast<void **>(&ix->d_tq_scale), size_t(dim) * sizeof(float)) != hipSuccess) {
+            hipMalloc(reinterpret_cast<void **>(&ix->d_tq_scale), size_t(dim) * sizeof(float)) != hipSuccess ||
+            hipMalloc(reinterpret_cast<void **>(&ix->d_tau_open), kTauOpenInts * sizeof(int)) != hipSuccess) {
+            rc = TV_ERR_HIP;
+            break;
+        }
+        // floors of a search's first sampling level: the order key of -inf for every query, written once
+        if (tv::launch_fill_i32(ix->d_tau_open, int(0x807fffffu), kTauOpenInts, ix->stream) != hipSuccess ||
+            hipStreamSynchronize(ix->stream) != hipSuccess) {
             rc = TV_ERR_HIP;
             break;
         }
@@ -506,7 +515,7 @@ int tv_index_destroy(tv_index *ix) {
     (void)hipSetDevice(ix->device);
     if (ix->stream) (void)hipStreamSynchronize(ix->stream);
     void *ptrs[] = {ix->d_signs, ix->d_perms, ix->d_centroids, ix->d_tq_shift, ix->d_tq_scale,
-                    ix->d_codes, ix->d_scales, ix->ws};
+                    ix->d_codes, ix->d_scales, ix->ws, ix->d_tau_open};
     for (void *p : ptrs) if (p) (void)hipFree(p);
     if (ix->stream) (void)hipStreamDestroy(ix->stream);
     delete ix;

@@ -144,6 +144,7 @@ struct tv_index {
     uint32_t *d_perms = nullptr;
     float *d_centroids = nullptr;
     float *d_tq_shift = nullptr, *d_tq_scale = nullptr;
+    int *d_tau_open = nullptr;     // order key of -inf per query: the floors before any level has run
 
     uint8_t *d_codes = nullptr;
     float *d_scales = nullptr;

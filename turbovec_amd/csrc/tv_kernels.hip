@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) void k_build_p(const float *__restrict__ qcal,
     }
     if (t == 0) {
         qscale[qi] = cs * qs;
-        qbias[qi] = 0.0f + bias_corr[qi];
+        qbias[qi] = 0.0f + (bias_corr ? bias_corr[qi] : 0.0f);
     }
 }
 
@@ -286,7 +286,7 @@ __global__ __launch_bounds__(256) void k_build_lut(const float *__restrict__ qca
         float bias = 0.0f;  // sequential f32 sum over groups, inner add first (search.rs:2910)
         for (int g = 0; g < G; ++g) bias += lut_lds[2 * g] + lut_lds[2 * g + 1];
         qscale[qi] = scale;
-        qbias[qi] = bias + bias_corr[qi];
+        qbias[qi] = bias + (bias_corr ? bias_corr[qi] : 0.0f);
     }
     for (int g = t; g < nch * 32; g += 256) {
         uint32_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -958,14 +958,16 @@ __global__ __launch_bounds__(256) void k_merge(const float *__restrict__ part_sc
 // redo through the list path.
 // ===========================================================================
 
-__global__ __launch_bounds__(256) void k_final(const uint64_t *__restrict__ cand,
+constexpr int kFinalThreads = 1024;
+
+__global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restrict__ cand,
                                                const uint32_t *__restrict__ cand_cnt, uint32_t n_seg,
                                                uint32_t seg_stride, int k_eff, int k_floor,
                                                float *__restrict__ out_scores, int64_t *__restrict__ out_idx,
                                                uint32_t *__restrict__ overflow, int *__restrict__ tau_out,
                                                int tau_stride_q) {
     __shared__ uint64_t keys[kFinalCap];
-    __shared__ uint32_t wave_sum[4];
+    __shared__ uint32_t wave_sum[kFinalThreads / 64];
     __shared__ uint32_t any_full;
     const int qn = blockIdx.x;
     const int t = threadIdx.x;
@@ -974,7 +976,7 @@ __global__ __launch_bounds__(256) void k_final(const uint64_t *__restrict__ cand
     if (t == 0) any_full = 0u;
     __syncthreads();
     // every thread owns a contiguous run of this query's segments
-    const uint32_t per = (n_seg + 255) / 256;
+    const uint32_t per = (n_seg + kFinalThreads - 1) / kFinalThreads;
     const uint32_t s0 = min(uint32_t(t) * per, n_seg), s1 = min(s0 + per, n_seg);
     const uint32_t *cnt = cand_cnt + size_t(qn) * seg_stride;
     uint32_t mine = 0;
@@ -992,11 +994,12 @@ __global__ __launch_bounds__(256) void k_final(const uint64_t *__restrict__ cand
     if ((t & 63) == 63) wave_sum[t >> 6] = incl;
     __syncthreads();
     uint32_t base = incl - mine, total = 0;
-    for (int w = 0; w < 4; ++w) { if (w < (t >> 6)) base += wave_sum[w]; total += wave_sum[w]; }
+    for (int w = 0; w < kFinalThreads / 64; ++w) { if (w < (t >> 6)) base += wave_sum[w]; total += wave_sum[w]; }
     const bool too_many = total > uint32_t(kFinalCap);
-    if (!sampling && (too_many || any_full || total < uint32_t(k_eff))) {
-        if (t == 0) overflow[qn] = 1u;     // the caller redoes this query through the list path
-        return;
+    if (!sampling) {
+        const bool redo = too_many || any_full || total < uint32_t(k_eff);
+        if (t == 0) overflow[qn] = redo ? 1u : 0u;   // set: the caller redoes this query through the exact path
+        if (redo) return;
     }
     if (sampling && total < uint32_t(k_eff)) {
         if (t == 0) *tau_slot = kTauInit;  // too few allowed slots sampled: the floor stays open
@@ -1014,11 +1017,11 @@ __global__ __launch_bounds__(256) void k_final(const uint64_t *__restrict__ cand
     uint32_t sort_n = 2;
     while (sort_n < c_all) sort_n <<= 1;
     __syncthreads();
-    for (uint32_t i = c_all + t; i < sort_n; i += 256) keys[i] = 0ull;
+    for (uint32_t i = c_all + t; i < sort_n; i += kFinalThreads) keys[i] = 0ull;
     __syncthreads();
     for (uint32_t size = 2; size <= sort_n; size <<= 1) {
         for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
-            for (uint32_t i = t; i < sort_n / 2; i += 256) {
+            for (uint32_t i = t; i < sort_n / 2; i += kFinalThreads) {
                 const uint32_t lo = 2 * i - (i & (stride - 1));
                 const uint32_t hi = lo + stride;
                 const bool desc = (lo & size) == 0;
@@ -1038,7 +1041,7 @@ __global__ __launch_bounds__(256) void k_final(const uint64_t *__restrict__ cand
         }
         return;
     }
-    for (int jj = t; jj < k_eff; jj += 256) {
+    for (int jj = t; jj < k_eff; jj += kFinalThreads) {
         float s; uint32_t idx;
         sort_unkey(keys[jj], s, idx);
         out_scores[size_t(qn) * k_eff + jj] = s;
@@ -1306,7 +1309,7 @@ hipError_t launch_final(const uint64_t *cand, const uint32_t *cand_cnt, uint32_t
                         int k_eff, int k_floor, int nq, float *out_scores, int64_t *out_idx, uint32_t *overflow,
                         int *tau_out, int tau_stride_q, hipStream_t s) {
     if (nq == 0 || k_eff == 0) return hipSuccess;
-    hipLaunchKernelGGL(k_final, dim3(nq), dim3(256), 0, s, cand, cand_cnt, n_seg, seg_stride, k_eff, k_floor,
+    hipLaunchKernelGGL(k_final, dim3(nq), dim3(kFinalThreads), 0, s, cand, cand_cnt, n_seg, seg_stride, k_eff, k_floor,
                        out_scores, out_idx, overflow, tau_out, tau_stride_q);
     return hipGetLastError();
 }
