@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Search-throughput benchmark of the HIP path: queries/s and achieved HBM GB/s.
 
-Workload (BASELINE.json's metric): TurboQuantIndex 10,000,000 x 1536, 4-bit,
+Workload (the headline metric): TurboQuantIndex 10,000,000 x 1536, 4-bit,
 k=10, no filter.  One step = one batch search (default 1024 queries) over the
 whole index, with the index, the queries and the result buffers already
 resident in HBM when the timed region starts.  A batch-1 figure is measured in
