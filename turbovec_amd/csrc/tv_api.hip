@@ -288,7 +288,7 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
 // the last one being 1 (the full scan).  The first level reads about `first`
 // slots and, having no floor yet, appends all of them (one short sort); level
 // sizes then grow geometrically to the full index, by a factor chosen so that
-// a level filtered by the floor of the one before appends at most about 2048
+// a level filtered by the floor of the one before appends at most about 4096
 // candidates per query (the floor is the k_floor-th best of the level before,
 // so a level `ratio` times larger keeps about ratio * k_floor).  The sampling
 // levels together read about 1/ratio of the index.
@@ -297,7 +297,7 @@ std::vector<uint32_t> sampling_steps(size_t n_blocks, size_t k_floor) {
     const double first = double(std::max<size_t>(1024, 8 * k_floor));
     std::vector<uint32_t> steps;
     if (n_slots > 2.0 * first) {
-        const double max_ratio = std::max(4.0, 2048.0 / double(k_floor));
+        const double max_ratio = std::max(4.0, double(tv::kFinalCap / 2) / double(k_floor));
         const int levels = std::max(1, int(std::ceil(std::log(n_slots / first) / std::log(max_ratio))));
         const double ratio = std::pow(n_slots / first, 1.0 / double(levels));
         double sample = first;
