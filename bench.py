@@ -146,17 +146,19 @@ def main():
             launches += nl
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        return dt, scan_ms, launches
+        return dt, scan_ms, launches, ix.queries_per_launch()
 
     alg_bytes = n_blocks * G * 32 + 4 * n          # codes + per-vector scales, one pass
     d_codes, _, code_bytes = ix.device_ptrs()
     read_ms = ix.stream_probe(d_codes, None, code_bytes, reps=5)   # pure read of the same buffer
     read_probe = code_bytes / (read_ms * 1e-3) / 1e9
-    dt, scan_ms, launches = run(args.batch, args.steps, args.warmup)
+    dt, scan_ms, launches, q_full = run(args.batch, args.steps, args.warmup)
+    # a step is ceil(batch / q_full) full-scan launches; the last may serve fewer queries
+    q_per_launch = args.batch / max(1, -(-args.batch // max(q_full, 1)))
     value = args.batch * args.steps / dt
     launch_s = scan_ms * 1e-3 / max(launches, 1)
     achieved = alg_bytes / launch_s / 1e9
-    dt1, scan1_ms, launches1 = run(1, max(args.steps, 15), args.warmup)
+    dt1, scan1_ms, launches1, _ = run(1, max(args.steps, 15), args.warmup)
     b1_steps = max(args.steps, 15)
     b1_launch_s = scan1_ms * 1e-3 / max(launches1, 1)
 
@@ -178,9 +180,8 @@ def main():
     host_single_s = median_host_call(q_host[:1], 15)
     host_qps = args.batch / host_batch_s
 
-    q_per_launch = args.batch * args.steps / max(launches, 1)
     if mode_p:
-        kernel = "k_scan_p4_multi" if q_per_launch > 32 else "k_scan_p4"
+        kernel = "k_scan_p4_multi" if q_full > 32 else "k_scan_p4"
     else:
         kernel = "k_scan_lut"
     traffic = MEASURED_TRAFFIC.get((kernel, n, dim, bits))
@@ -215,7 +216,8 @@ def main():
                      "kernel": kernel,
                      "achievable_read_GBps": read_probe, "frac_of_achievable": achieved / read_probe,
                      "algorithmic_bytes_per_launch": alg_bytes, "launches_timed": launches,
-                     "mean_launch_ms": launch_s * 1e3, "queries_per_launch": q_per_launch},
+                     "mean_launch_ms": launch_s * 1e3, "queries_per_launch": q_per_launch,
+                     "queries_per_full_launch": q_full},
     }
     if mode_p:
         out["mfma"] = {"achieved": int8_ops / launch_s / 1e12, "peak": 5000.0, "unit": "TOP/s",

@@ -194,6 +194,8 @@ int tv_debug_prepare(tv_index *ix, const float *queries, size_t nq,
  * tv_search* call on this index, measured with HIP events on its stream, and
  * how many launches that was. */
 int tv_last_scan_ms(const tv_index *ix, float *ms, int *launches);
+/* Queries one full-scan launch of the last search served (a full launch of a large batch). */
+int tv_debug_queries_per_launch(const tv_index *ix, int *queries);
 /* Path selection for tests (results must be identical either way): bit 0 makes
  * every search take the full-range list / dense-select path instead of
  * sample-then-filter; bit 1 keeps large batches on the one-tile-per-launch scan

@@ -29,7 +29,7 @@ EXPORTS = [
     "tv_index_set_calibration", "tv_index_set_score_mode", "tv_index_get_tables", "tv_index_upload_seq",
     "tv_index_upload_seq_dev", "tv_index_append_rows", "tv_index_add", "tv_index_add_dev", "tv_index_calibrate", "tv_index_get_calibration", "tv_index_swap_remove", "tv_index_download_seq", "tv_index_len", "tv_index_dim",
     "tv_index_bits", "tv_validate_queries", "tv_pack_mask", "tv_search", "tv_search_dev", "tv_debug_scan",
-    "tv_debug_prepare", "tv_last_scan_ms", "tv_index_device_ptrs", "tv_host_rotation_tables", "tv_host_codebook",
+    "tv_debug_prepare", "tv_last_scan_ms", "tv_debug_queries_per_launch", "tv_index_device_ptrs", "tv_host_rotation_tables", "tv_host_codebook",
     "tv_debug_stream_probe", "tv_debug_set_path", "tv_debug_overflow_redos",
     "tv_host_snapshot_len", "tv_host_snapshot_compose", "tv_host_snapshot_info", "tv_host_snapshot_extract",
     "tv_index_to_bytes", "tv_index_from_bytes",
@@ -91,6 +91,7 @@ def lib():
     L.tv_debug_scan.argtypes = [vp, vp, sz, vp, vp]
     L.tv_debug_prepare.argtypes = [vp, vp, sz, vp, vp, vp]
     L.tv_last_scan_ms.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(i32)]
+    L.tv_debug_queries_per_launch.argtypes = [vp, C.POINTER(i32)]
     L.tv_index_device_ptrs.argtypes = [vp, C.POINTER(vp), C.POINTER(vp), C.POINTER(sz)]
     L.tv_debug_set_path.argtypes = [vp, i32]
     L.tv_debug_overflow_redos.argtypes = [vp, C.POINTER(sz)]
@@ -278,6 +279,11 @@ class NativeIndex:
         n = C.c_int(0)
         check(lib().tv_last_scan_ms(self.h, C.byref(ms), C.byref(n)))
         return ms.value, n.value
+
+    def queries_per_launch(self):
+        n = C.c_int(0)
+        check(lib().tv_debug_queries_per_launch(self.h, C.byref(n)))
+        return n.value
 
     def set_path(self, force_full_lists):
         check(lib().tv_debug_set_path(self.h, int(force_full_lists)))

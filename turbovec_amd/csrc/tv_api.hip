@@ -379,6 +379,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             const int lgrid = int(std::min<size_t>(size_t(grid), std::max<size_t>(1, (level_blocks + 1) / 2)));
             const bool batched = nt_batched > 0;
             const size_t tiles_per_launch = batched ? size_t(nt_batched) : 1;
+            ix->last_queries_per_launch = int(std::min(cq, tile_q * tiles_per_launch));
             int n_seg = lgrid;
             size_t launch_no = 0;
             for (size_t t = 0; t < n_tiles; t += tiles_per_launch, ++launch_no) {
@@ -1101,6 +1102,12 @@ int tv_debug_set_path(tv_index *ix, int force_full_lists) {
 int tv_debug_overflow_redos(const tv_index *ix, size_t *count) {
     if (!ix || !count) return TV_ERR_BAD_ARGUMENT;
     *count = ix->overflow_redos;
+    return TV_OK;
+}
+
+int tv_debug_queries_per_launch(const tv_index *ix, int *queries) {
+    if (!ix || !queries) return TV_ERR_BAD_ARGUMENT;
+    *queries = ix->last_queries_per_launch;
     return TV_OK;
 }
 

@@ -157,6 +157,7 @@ struct tv_index {
     size_t ws_bytes = 0;
     float last_scan_ms = 0.0f;
     int last_scan_launches = 0;
+    int last_queries_per_launch = 0;   // queries one full-scan launch of the last search served
     int force_robust = 0;          // test hook: skip sample-then-filter
     int no_batched = 0;            // test hook: one query tile per scan launch even for large batches
     size_t overflow_redos = 0;     // queries redone because their candidate buffer overflowed
