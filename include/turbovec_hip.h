@@ -199,7 +199,8 @@ int tv_debug_queries_per_launch(const tv_index *ix, int *queries);
 /* Path selection for tests (results must be identical either way): bit 0 makes
  * every search take the full-range list / dense-select path instead of
  * sample-then-filter; bit 1 keeps large batches on the one-tile-per-launch scan
- * instead of the batched one. */
+ * instead of the batched ones; bit 2 keeps them off the all-queries-per-pass
+ * kernel only. */
 int tv_debug_set_path(tv_index *ix, int force_full_lists);
 /* How many queries so far had to be redone through that path because their
  * candidate buffer overflowed. */

@@ -1,0 +1,83 @@
+"""The wide permute-dot scan (every query of a chunk in one pass over the codes) against the
+CPU oracle and against the tile-group kernels it replaces for large high-dimensional
+batches.  Bar: slots and float scores bit-exact."""
+import numpy as np
+import pytest
+
+from helpers import OracleIndex, bits_equal, to_native, unit_gaussian
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def T():
+    from turbovec_amd import _lib
+    _lib.lib()
+    return _lib
+
+
+def masks_for(T, n, seed):
+    rng = np.random.default_rng(seed)
+    out = [None, rng.random(n) < 0.5, rng.random(n) < 0.004, (np.arange(n) >= n // 3) & (np.arange(n) < n // 3 + 700)]
+    return [None if m is None else T.pack_mask(m)[0] for m in out]
+
+
+# dims 1536 and 1280 switch to the wide kernel at 256 queries, 1024 at 512; the query counts
+# leave a ragged last tile, and 1029 = one full chunk of 1024 plus a 5-query chunk that the
+# single-tile kernel serves
+@pytest.mark.parametrize("dim,n,nq", [(1536, 6_007, 300), (1280, 4_001, 257), (1024, 5_003, 520), (1536, 3_001, 1029)])
+def test_wide_scan_matches_oracle(T, oracle, dim, n, nq):
+    oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=dim + n))
+    q = unit_gaussian(nq, dim, seed=77)
+    ix = to_native(T, oidx)
+    for words in masks_for(T, n, 8):
+        for k in (1, 10, 100):
+            s, i = ix.search(q, k, mask_words=words)
+            assert ix.queries_per_launch() >= 256 or nq == 1029
+            os_, oi = oidx.search(q, k, mask_words=words)
+            assert np.array_equal(i, oi), k
+            assert bits_equal(s, os_), k
+    ix.close()
+
+
+def test_wide_launch_covers_the_chunk(T, oracle):
+    """The library reports how many queries its last full-scan launch served: the whole
+    chunk on the wide path, at most a group of tiles with the wide path switched off."""
+    oidx = OracleIndex(oracle, 1536, 4, unit_gaussian(2_000, 1536, seed=5))
+    ix = to_native(T, oidx)
+    q = unit_gaussian(512, 1536, seed=6)
+    ix.search(q, 10)
+    assert ix.queries_per_launch() == 512
+    ix.set_path(4)
+    ix.search(q, 10)
+    assert ix.queries_per_launch() < 512
+    ix.close()
+
+
+# device-encoded index too large for the oracle: the wide kernel against the tile-group
+# kernels and the exact full-list path on the same index (k up to the sort capacity's regime)
+@pytest.mark.parametrize("dim,n,nq", [(1536, 300_000, 1024 + 300), (1024, 200_000, 700)])
+def test_wide_scan_matches_other_paths(T, dim, n, nq):
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(dim)
+    ix = T.NativeIndex(dim, 4)
+    for c0 in range(0, n, 100_000):
+        v = torch.randn(min(100_000, n - c0), dim, device=dev, generator=gen)
+        torch.cuda.synchronize()
+        ix.add_dev(v.data_ptr(), v.shape[0])
+    q = torch.randn(nq, dim, device=dev, generator=gen).cpu().numpy()
+    for words in masks_for(T, n, 9):
+        for k in (10, 1000):
+            s, i = ix.search(q, k, mask_words=words)
+            ix.set_path(4)
+            s2, i2 = ix.search(q, k, mask_words=words)
+            ix.set_path(0)
+            assert np.array_equal(i, i2) and bits_equal(s, s2), k
+        ix.set_path(1)
+        s3, i3 = ix.search(q[:40], 10, mask_words=words)
+        ix.set_path(0)
+        s, i = ix.search(q, 10, mask_words=words)
+        assert np.array_equal(i[:40], i3) and bits_equal(s[:40], s3)
+    ix.close()

@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libturbovec_hip.so")
 
-SOURCES = ["tv_kernels.hip", "tv_kernels2.hip", "tv_encode.hip", "tv_api.hip", "host_tables.cpp", "tv_snapshot.cpp"]
+SOURCES = ["tv_kernels.hip", "tv_kernels2.hip", "tv_kernels3.hip", "tv_encode.hip", "tv_api.hip", "host_tables.cpp", "tv_snapshot.cpp"]
 
 # -ffp-contract=off: the parity contract is bit-exact float arithmetic, fused
 # only where the code says fmaf.  The packed-FP32 feature is switched off for

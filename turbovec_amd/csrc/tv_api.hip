@@ -349,7 +349,11 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
         const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_append_queries(g.nch));
         const size_t n_tiles = (cq + tile_q - 1) / tile_q;
         const size_t cq_pad = n_tiles * tile_q;
-        const int grid = mode_p ? tv::scan_grid_blocks(ix->device, mode_p, g.nch, 0, int(tile_q))
+        // large chunks of high-dimensional queries take the wide kernel: all of them in one pass per level
+        const int wide_min = tv::wide_min_queries(g.nch);
+        const bool wide = mode_p && !ix->no_batched && !ix->no_wide && wide_min > 0 && cq >= size_t(wide_min);
+        const int grid = wide ? tv::wide_grid_blocks(ix->device)
+                       : mode_p ? tv::scan_grid_blocks(ix->device, mode_p, g.nch, 0, int(tile_q))
                                 : tv::lut_append_grid(ix->device, g.nch);
         const size_t seg_stride = size_t(grid);
         size_t need = prepare_bytes(ix, cq) + round_up(n_tiles * tv::kQTile * 4, 256) +
@@ -377,8 +381,8 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             const size_t level_blocks = (n_blocks + steps[lv] - 1) / steps[lv];
             // level 1 appends every slot it reads: two blocks per workgroup fill a segment exactly
             const int lgrid = int(std::min<size_t>(size_t(grid), std::max<size_t>(1, (level_blocks + 1) / 2)));
-            const bool batched = nt_batched > 0;
-            const size_t tiles_per_launch = batched ? size_t(nt_batched) : 1;
+            const bool batched = nt_batched > 0 && !wide;
+            const size_t tiles_per_launch = wide ? n_tiles : batched ? size_t(nt_batched) : 1;
             ix->last_queries_per_launch = int(std::min(cq, tile_q * tiles_per_launch));
             int n_seg = lgrid;
             size_t launch_no = 0;
@@ -398,7 +402,10 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
                 a.seg_stride = uint32_t(seg_stride);
                 const bool timed = last && int(launch_no) < kMaxTimedTiles;
                 if (timed) TV_HIP(hipEventRecord(g_events.start[launch_no], ix->stream));
-                if (batched) {
+                if (wide) {
+                    n_seg = grid;
+                    TV_HIP(tv::launch_scan_p4_wide(a, n_seg, ix->stream));
+                } else if (batched) {
                     n_seg = int(std::min<size_t>(size_t(bgrid), seg_stride));
                     TV_HIP(tv::launch_scan_p4_batched(a, n_seg, ix->stream));
                 } else if (mode_p) {
@@ -1096,6 +1103,7 @@ int tv_debug_set_path(tv_index *ix, int force_full_lists) {
     if (!ix) return TV_ERR_BAD_ARGUMENT;
     ix->force_robust = (force_full_lists & 1) != 0;
     ix->no_batched = (force_full_lists & 2) != 0;
+    ix->no_wide = (force_full_lists & 4) != 0;
     return TV_OK;
 }
 

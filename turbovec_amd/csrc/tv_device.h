@@ -84,4 +84,55 @@ __device__ __forceinline__ void sort_unkey(uint64_t key, float &s, uint32_t &idx
 }
 
 
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// ---------------------------------------------------------------------------
+// Hand-placed code loads.  The vector-memory counter retires in order, and the
+// compiler's own wait placement is decided per merge point of the control flow,
+// which for a software-pipelined stream ends up waiting on the burst it has
+// just issued.  These loads are invisible to that pass: the kernel states how
+// many younger loads may stay in flight where it consumes a register
+// (wait_vm<N>).  Loads the compiler issues itself only make its own waits
+// stricter, never looser, because a count is an upper bound on what may remain.
+// ---------------------------------------------------------------------------
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <int OFF>
+__device__ __forceinline__ void load16_async(u32x4 &dst, const void *p) {
+    asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(dst) : "v"(p), "n"(OFF));
+}
+__device__ __forceinline__ void load4_async(float &dst, const void *p) {
+    asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(p));
+}
+template <int N>
+__device__ __forceinline__ void wait_vm(u32x4 &r) {
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(r) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_vm(float &r) {
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(r) : "n"(N));
+}
+
+// Four packed nibbles (one per byte, values 0..15) -> four int8 levels.
+// v_perm_b32 looks up 8 table bytes; selectors >= 13 give 0xff, so each half
+// of the 16-entry table is looked up with the other half's nibbles pushed out
+// of range, and the two results are ANDed.
+__device__ __forceinline__ uint32_t levels_of(uint32_t nib, uint32_t t0, uint32_t t1, uint32_t t2, uint32_t t3) {
+    const uint32_t selA = nib + (nib & 0x08080808u);  // 0..7 stay, 8..15 -> 16..23
+    const uint32_t selB = selA ^ 0x10101010u;         // 0..7 -> 16..23, 16..23 -> 0..7
+    return __builtin_amdgcn_perm(t1, t0, selA) & __builtin_amdgcn_perm(t3, t2, selB);
+}
+
+
+// Compile-time loop: f(IntC<0>{}), ..., f(IntC<N-1>{}), for bodies that index register arrays.
+template <int V> struct IntC { static constexpr int value = V; };
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(IntC<I>{});
+        static_for<N, I + 1>(f);
+    }
+}
+
 }  // namespace tv

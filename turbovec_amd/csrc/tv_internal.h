@@ -108,6 +108,11 @@ int batched_grid_blocks(int device, int nch);
 hipError_t launch_scan_p4_batched(const ScanArgs &a, int grid, hipStream_t s);
 // out_tau == nullptr: write the k_eff best of the merged lists; else write only the
 // order key of the k_eff-th best (a floor at least k_eff scanned slots reach) per query.
+// Wide batched scan (every query of a chunk in one pass; tv_kernels3.hip).
+int wide_min_queries(int nch);
+int wide_grid_blocks(int device);
+hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s);
+
 hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, const int *part_cnt, int total_threads,
                         int qmod, int k, int k_eff, int nq_tile, float *out_scores, int64_t *out_idx,
                         int *out_tau, hipStream_t s);
@@ -160,5 +165,6 @@ struct tv_index {
     int last_queries_per_launch = 0;   // queries one full-scan launch of the last search served
     int force_robust = 0;          // test hook: skip sample-then-filter
     int no_batched = 0;            // test hook: one query tile per scan launch even for large batches
+    int no_wide = 0;               // test hook: large batches go through the tile-group kernels, not the wide one
     size_t overflow_redos = 0;     // queries redone because their candidate buffer overflowed
 };

@@ -23,8 +23,6 @@ namespace tv {
 // ===========================================================================
 
 typedef uint32_t lut_u32x2 __attribute__((ext_vector_type(2)));
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
 
 // base + byte E of packed, in one instruction (sub-dword operand select).
 template <int E>
@@ -53,7 +51,6 @@ __device__ __forceinline__ v4i lut_a_operand<1, uint8_t>(const uint8_t (&)[16], 
 template <>
 __device__ __forceinline__ v4i lut_a_operand<2, uint16_t>(const uint16_t (&)[16], int) { return v4i{0, 0, 0, 0}; }
 
-template <int V> struct IntC { static constexpr int value = V; };
 template <typename F>
 __device__ __forceinline__ void static_for4(F &&f) { f(IntC<0>{}); f(IntC<1>{}); f(IntC<2>{}); f(IntC<3>{}); }
 
