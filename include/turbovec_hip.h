@@ -210,6 +210,14 @@ int tv_debug_overflow_redos(const tv_index *ix, size_t *count);
  * milliseconds per launch.  Calibrates the achievable HBM rate and gives the
  * hardware counters a kernel of known traffic. */
 int tv_debug_stream_probe(tv_index *ix, const void *d_src, void *d_dst, size_t bytes, int reps, float *ms_per_rep);
+/* Matrix-unit probe on the index's stream: reps launches of the batched scan's
+ * MFMA loop alone (int8 32x32x32, A operands in registers, B operands read from
+ * LDS, pseudo-random bytes, no HBM traffic), iters x 48 MFMAs per wavefront;
+ * mean milliseconds per launch and the int8 operations (2 per multiply-add) of
+ * one launch.  Calibrates the rate the matrix unit sustains on this chip under
+ * its power management, as the read probe does for HBM.  No counterpart in the
+ * reference (its roofline probe is the read one, examples/stream_bw.rs:30-66). */
+int tv_debug_mfma_probe(tv_index *ix, int iters, int reps, float *ms_per_rep, double *ops_per_rep);
 /* Device pointers of the resident index (native layout) for tools. */
 int tv_index_device_ptrs(const tv_index *ix, void **d_codes, void **d_scales, size_t *code_bytes);
 

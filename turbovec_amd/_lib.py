@@ -30,7 +30,7 @@ EXPORTS = [
     "tv_index_upload_seq_dev", "tv_index_append_rows", "tv_index_add", "tv_index_add_dev", "tv_index_calibrate", "tv_index_get_calibration", "tv_index_swap_remove", "tv_index_download_seq", "tv_index_len", "tv_index_dim",
     "tv_index_bits", "tv_validate_queries", "tv_pack_mask", "tv_search", "tv_search_dev", "tv_debug_scan",
     "tv_debug_prepare", "tv_last_scan_ms", "tv_debug_queries_per_launch", "tv_index_device_ptrs", "tv_host_rotation_tables", "tv_host_codebook",
-    "tv_debug_stream_probe", "tv_debug_set_path", "tv_debug_overflow_redos",
+    "tv_debug_stream_probe", "tv_debug_mfma_probe", "tv_debug_set_path", "tv_debug_overflow_redos",
     "tv_host_snapshot_len", "tv_host_snapshot_compose", "tv_host_snapshot_info", "tv_host_snapshot_extract",
     "tv_index_to_bytes", "tv_index_from_bytes",
 ]
@@ -96,6 +96,7 @@ def lib():
     L.tv_debug_set_path.argtypes = [vp, i32]
     L.tv_debug_overflow_redos.argtypes = [vp, C.POINTER(sz)]
     L.tv_debug_stream_probe.argtypes = [vp, vp, vp, sz, i32, C.POINTER(C.c_float)]
+    L.tv_debug_mfma_probe.argtypes = [vp, i32, i32, C.POINTER(C.c_float), C.POINTER(C.c_double)]
     L.tv_host_rotation_tables.argtypes = [i32, vp, vp, C.POINTER(i32), C.POINTER(C.c_float)]
     L.tv_host_codebook.argtypes = [i32, i32, vp, vp]
     _lib = L
@@ -292,6 +293,12 @@ class NativeIndex:
         c = C.c_size_t(0)
         check(lib().tv_debug_overflow_redos(self.h, C.byref(c)))
         return c.value
+
+    def mfma_probe(self, iters=2000, reps=3):
+        """int8 operations per second of the batched scan's MFMA loop alone (registers x LDS, no HBM)."""
+        ms, ops = C.c_float(0), C.c_double(0)
+        check(lib().tv_debug_mfma_probe(self.h, iters, reps, C.byref(ms), C.byref(ops)))
+        return ops.value / (ms.value * 1e-3)
 
     def stream_probe(self, d_src_ptr, d_dst_ptr, nbytes, reps=5):
         """Mean ms per launch of a read-sum (d_dst_ptr None) or copy kernel over nbytes."""

@@ -1099,6 +1099,28 @@ int tv_debug_stream_probe(tv_index *ix, const void *d_src, void *d_dst, size_t b
     return TV_OK;
 }
 
+int tv_debug_mfma_probe(tv_index *ix, int iters, int reps, float *ms_per_rep, double *ops_per_rep) {
+    if (!ix || iters <= 0 || reps <= 0) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    int rc = ensure_events();
+    if (rc != TV_OK) return rc;
+    rc = ensure_workspace(ix, 4096);
+    if (rc != TV_OK) return rc;
+    uint32_t *sink = static_cast<uint32_t *>(ix->ws);
+    double ops = 0.0;
+    TV_HIP(tv::launch_probe_mfma(ix->device, iters, sink, &ops, ix->stream));  // warm
+    TV_HIP(hipEventRecord(g_events.start[0], ix->stream));
+    for (int r = 0; r < reps; ++r) TV_HIP(tv::launch_probe_mfma(ix->device, iters, sink, &ops, ix->stream));
+    TV_HIP(hipEventRecord(g_events.stop[0], ix->stream));
+    TV_HIP(hipStreamSynchronize(ix->stream));
+    float ms = 0.0f;
+    TV_HIP(hipEventElapsedTime(&ms, g_events.start[0], g_events.stop[0]));
+    if (ms_per_rep) *ms_per_rep = ms / float(reps);
+    if (ops_per_rep) *ops_per_rep = ops;
+    return TV_OK;
+}
+
 int tv_debug_set_path(tv_index *ix, int force_full_lists) {
     if (!ix) return TV_ERR_BAD_ARGUMENT;
     ix->force_robust = (force_full_lists & 1) != 0;

@@ -125,6 +125,7 @@ hipError_t launch_final(const uint64_t *cand, const uint32_t *cand_cnt, uint32_t
                         int *tau_out, int tau_stride_q, hipStream_t s);
 hipError_t launch_fill_i32(int *p, int v, size_t n, hipStream_t s);
 hipError_t launch_probe(const void *src, void *dst, size_t bytes, int copy, uint32_t *sink, hipStream_t s);
+hipError_t launch_probe_mfma(int device, int iters, uint32_t *sink, double *ops, hipStream_t s);
 // Exact top-k of a dense score row per query (NaN = excluded slot).
 hipError_t launch_select_topk(const float *d_scores, size_t n, int nq_tile, size_t k_eff, uint64_t *d_keys_tmp,
                               uint32_t *d_hist, float *out_scores, int64_t *out_idx, hipStream_t s);

@@ -250,6 +250,58 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
     for (int q = tid; q < nq; q += kWideThreads) a.cand_cnt[size_t(q) * a.seg_stride + blockIdx.x] = sq[q].cnt;
 }
 
+// Matrix-unit probe: the wide kernel's MFMA loop alone -- A operands resident in registers,
+// B operands read from LDS, pseudo-random bytes in both (operand toggling sets the power
+// the clock is managed against) -- with no HBM traffic, no barriers and no epilogue.  Its rate
+// is what this loop shape can sustain on the chip at hand; the nominal peak assumes the top clock.
+__global__ __launch_bounds__(kWideThreads, 2) void k_probe_mfma(int iters, uint32_t *sink) {
+    constexpr int NCH = 24, NB = 2;
+    extern __shared__ __align__(16) uint8_t smem[];
+    for (uint32_t i = threadIdx.x; i < NCH * 1024 / 4; i += kWideThreads)
+        reinterpret_cast<uint32_t *>(smem)[i] = (i * 2654435761u) ^ ((i * 40503u) << 13) ^ ((i >> 3) * 97u);
+    __syncthreads();
+    const uint32_t baddr = uint32_t(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)smem)) +
+                           (threadIdx.x & 63) * 16;
+    v4i alo[NCH], ahi[NCH];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        uint32_t x = (threadIdx.x * 64 + c) * 2654435761u;
+        alo[c] = v4i{int(x), int(x * 31u + 7u), int((x * 131u) ^ 0x5bd1e995u), int(x * 1664525u + 1013904223u)};
+        x ^= 0x9e3779b9u;
+        ahi[c] = v4i{int(x * 17u), int(x * 31u + 9u), int((x * 137u) ^ 0x5bd1e995u), int(x * 22695477u + 1u)};
+    }
+    v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    for (int it = 0; it < iters; ++it) {
+        static_for<2>([&](auto hh) {
+            constexpr int c0 = decltype(hh)::value * (NCH / 2);
+            v4i w[NB];
+            static_for<NB>([&](auto mm) { lds_read16_async<decltype(mm)::value * 1024>(w[decltype(mm)::value], baddr); });
+            static_for<NCH>([&](auto mm) {
+                constexpr int m = decltype(mm)::value;
+                constexpr int younger = NCH - 1 - m < NB - 1 ? NCH - 1 - m : NB - 1;
+                lds_wait<younger>(w[m % NB]);
+                if constexpr ((m & 1) == 0)
+                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo[c0 + m / 2], w[m % NB], acc, 0, 0, 0);
+                else
+                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi[c0 + m / 2], w[m % NB], acc, 0, 0, 0);
+                if constexpr (m + NB < NCH) lds_read16_async<(m + NB) * 1024>(w[m % NB], baddr);
+            });
+        });
+    }
+    uint32_t x = 0;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) x ^= uint32_t(acc[r]);
+    if (x == 0x9e3779b9u && iters < 0) sink[0] = x;   // keeps the loop alive; never taken
+}
+
+// One launch of the probe on every CU; *ops = int8 operations (2 per multiply-add) it performs.
+hipError_t launch_probe_mfma(int device, int iters, uint32_t *sink, double *ops, hipStream_t s) {
+    const int grid = wide_grid_blocks(device);
+    hipLaunchKernelGGL(k_probe_mfma, dim3(grid), dim3(kWideThreads), 24 * 1024, s, iters, sink);
+    if (ops) *ops = double(grid) * kWideWaves * double(iters) * 48.0 * 65536.0;
+    return hipGetLastError();
+}
+
 // Smallest chunk of queries the wide kernel is the faster one for (measured against the
 // tile-group kernels on 4-bit indexes of 1024, 1280 and 1536 dimensions); 0 = never.  Below
 // 1024 dimensions a tile is too few MFMAs for its two barriers and its epilogue.
