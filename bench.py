@@ -53,6 +53,9 @@ def parse():
     ap.add_argument("--score-mode", choices=["auto", "lut"], default="auto",
                     help="auto = what the reference runs on a VNNI/dotprod host (int8 permute-dot at 4-bit); "
                          "lut = the classic u8-LUT kernel's floats")
+    ap.add_argument("--tile-groups", action="store_true",
+                    help="keep large batches on the tile-group kernel (96 queries per pass over the codes) "
+                         "instead of the all-queries-per-pass one")
     ap.add_argument("--cpu-sample", type=int, default=2_000_000, help="vectors in the CPU-baseline sample (0 = skip)")
     ap.add_argument("--cpu-threads", type=int, default=16)
     ap.add_argument("--copy-probe", action="store_true",
@@ -121,6 +124,8 @@ def main():
     gen = torch.Generator(device=dev)
     gen.manual_seed(0)
     ix = T.NativeIndex(dim, bits)
+    if args.tile_groups:
+        ix.set_path(4)
     if args.score_mode == "lut":
         ix.set_score_mode(T.SCORE_L_CLASSIC)
     mode_p = bits == 4 and args.score_mode == "auto"
