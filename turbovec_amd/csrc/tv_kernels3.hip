@@ -47,9 +47,18 @@ __device__ __forceinline__ void lds_wait(v4i &r) {
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(r) : "n"(N));
 }
 
-struct WideQuery {          // per query, in LDS
-    float qs, qb, tau;      // tau is NaN for the padding queries of the last tile: nothing passes
+// Per query, in LDS.  A score is fmaf(float(acc), qs, qb) * row_scale and passes when it reaches
+// tau.  With tau, qs > 0 and row scales >= 0 that needs acc >= (tau / max_row_scale - qb) / qs, up
+// to rounding: ta / max_row_scale - tb is that bound in accumulator units with the roundings of
+// both sides priced in (relative 1e-5, against a few 2^-24, plus 2 for the integer conversions),
+// so comparing the largest accumulator of a lane with it never loses a candidate and lets the
+// common tile -- no candidate at all -- skip the float epilogue.
+struct WideQuery {
+    float ta, tb;           // ta = -inf: no such bound, always score (tau <= 0, open floor, odd qs); +inf: padding query
     uint32_t cnt;           // candidates this workgroup appended
+    float pad;
+    float qs, qb, tau;      // tau is NaN for the padding queries of the last tile: nothing passes
+    float pad2;
 };
 
 template <int NCH, int NB>
@@ -75,10 +84,17 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
     const uint32_t lane16 = uint32_t(lane) * 16;
     for (int q = tid; q < nq_pad; q += kWideThreads) {
         const bool act = q < nq;
-        sq[q].qs = act ? a.qscale[q] : 0.0f;
-        sq[q].qb = act ? a.qbias[q] : 0.0f;
-        sq[q].tau = act ? order_unkey(a.gtau[q]) : __int_as_float(0x7fc00000);
+        const float qs = act ? a.qscale[q] : 0.0f, qb = act ? a.qbias[q] : 0.0f;
+        const float tau = act ? order_unkey(a.gtau[q]) : __int_as_float(0x7fc00000);
+        sq[q].qs = qs;
+        sq[q].qb = qb;
+        sq[q].tau = tau;
         sq[q].cnt = 0u;
+        const float inf = __int_as_float(0x7f800000);
+        const bool bounded = tau > 0.0f && tau < inf && qs > 0.0f && qs < inf && fabsf(qb) < inf;
+        const float rb = qb / qs;
+        sq[q].ta = !act ? inf : bounded ? (tau / qs) * (1.0f - 1e-5f) : -inf;
+        sq[q].tb = act && bounded ? rb + 1e-5f * fabsf(rb) + 2.0f : 0.0f;
     }
     if (tid == 0) *snext = 0u;
     __syncthreads();
@@ -86,6 +102,12 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
     const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
     const uint32_t step = a.b_step;
     const uint32_t nj = (a.n_blocks + step - 1) / step;
+#ifdef WIDE_TIMING
+    unsigned long long tk[8] = {0, 0, 0, 0, 0, 0, 0, 0}, t_last = __builtin_readcyclecounter();
+#define TICK(i) { const unsigned long long now_ = __builtin_readcyclecounter(); tk[i] += now_ - t_last; t_last = now_; }
+#else
+#define TICK(i)
+#endif
 
     // next live block of this workgroup (blocks m * gridDim.x + blockIdx.x), claimed wave by wave
     auto claim = [&]() -> uint32_t {
@@ -102,9 +124,13 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
 
     // The weights are one periodic stream of slices (slice s = half s & 1 of tile s >> 1, kSlice
     // contiguous bytes; after the last tile the first follows again for the next round of blocks).
-    // Stream position g lives in ring slot g % kWideRing and is requested kAhead positions early, so
-    // behind the slice being consumed exactly (kAhead - 1) * kPieces of this wave's requests are
-    // younger -- the count its wait leaves outstanding (waves below kExtra request one piece more).
+    // Stream position g lives in ring slot g % kWideRing.  Half way through the MFMAs of slice g
+    // every wave waits for its own pieces of slice g + 1, meets the others at a barrier -- after
+    // which slice g + 1 is whole and slice g - 1 is read by nobody -- and requests slice g + 4 into
+    // the slot of g - 1.  The hand-over thus sits inside a run of MFMAs, where the SIMD's other wave
+    // keeps the matrix unit busy, and a wave that finishes slice g starts g + 1 without waiting.
+    // At that wait the requests for slices g + 2 and g + 3 are younger: 2 * pieces stay outstanding
+    // (waves below kExtra request one piece more).
     int req_slice = 0, req_slot = 0;                        // next stream position to request
     auto request_next = [&]() {
         const uint8_t *src = a.tables + size_t(req_slice) * kSlice + size_t(wave) * 1024;
@@ -117,18 +143,23 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
         req_slice = req_slice + 1 == n_slices ? 0 : req_slice + 1;
         req_slot = req_slot + 1 == kWideRing ? 0 : req_slot + 1;
     };
-    for (int i = 0; i < kAhead; ++i) request_next();
-    int use_slot = 0;                                       // ring slot of the slice consumed next
-
-    // Wait for the slice in use_slot, let everyone catch up, refill the slot freed by the previous
-    // slice, and return the consumed slice's B-operand address for this lane.
-    auto next_slice = [&]() -> uint32_t {
+    auto hand_over = [&](auto younger_slices) {
+        constexpr int ys = decltype(younger_slices)::value;
         if (kExtra != 0 && wave < kExtra)
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kAhead - 1) * (kPieces + 1)) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ys * (kPieces + 1)) : "memory");
         else
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kAhead - 1) * kPieces) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ys * kPieces) : "memory");
+        TICK(1)
         __syncthreads();
+        TICK(2)
         request_next();
+        TICK(3)
+    };
+    // slices 0..3 requested, slice 0 whole: the state the first hand-over expects
+    for (int i = 0; i < kAhead - 1; ++i) request_next();
+    hand_over(IntC<kAhead - 2>{});
+    int use_slot = 0;                                       // ring slot of the slice consumed next
+    auto slice_address = [&]() -> uint32_t {
         const uint32_t bp = lds_b + uint32_t(use_slot) * kSlice + lane16;
         use_slot = use_slot + 1 == kWideRing ? 0 : use_slot + 1;
         return bp;
@@ -138,7 +169,7 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
     v16i acc;
     // The NCH MFMAs of one slice.  MFMA m takes chunk HALF * NCH/2 + m/2 (low nibbles for even m,
     // high for odd) against the 1 KiB of weights at m * 1024, which come through NB registers
-    // requested NB MFMAs ahead.
+    // requested NB MFMAs ahead; the hand-over of the next slice sits in the middle.
     auto slice_mfmas = [&](auto half, uint32_t baddr) {
         constexpr int c0 = decltype(half)::value * (NCH / 2);
         v4i w[NB];
@@ -146,6 +177,10 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
         static_for<NCH>([&](auto mm) {
             constexpr int m = decltype(mm)::value;
             constexpr int younger = NCH - 1 - m < NB - 1 ? NCH - 1 - m : NB - 1;
+            if constexpr (m == NCH / 2) {
+                TICK(5)
+                hand_over(IntC<kAhead - 2>{});
+            }
             lds_wait<younger>(w[m % NB]);
             if constexpr ((m & 1) == 0)
                 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo[c0 + m / 2], w[m % NB], acc, 0, 0, 0);
@@ -155,11 +190,8 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
         });
     };
 
-    // Waves w and w + 4 share a SIMD and would otherwise reach their epilogues together with the
-    // MFMA pipe idle: the upper four score a tile one slice later, before the first MFMAs of
-    // the next tile, while the lower four already run theirs.
-    const bool late = wave >= kWideWaves / 2;
-
+    int inv_vmax = 0;        // bits of 1 / (largest allowed row scale of the block); +inf when that is 0
+    bool odd_block = false;
     for (;;) {
         // ---- block phase: claim, load, decode into registers ----
         const uint32_t j = claim();
@@ -187,37 +219,35 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
                     }
                 });
             });
-            if (lane < 32) {
-                const uint32_t slot = b * 32u + uint32_t(lane);
-                bool ok = slot < a.n;
-                if (ok && a.mask != nullptr) ok = (uint32_t(a.mask[b >> 1] >> ((b & 1) * 32)) >> lane) & 1u;
-                s_vs[wave * 32 + lane] = ok ? a.scales[slot] : __int_as_float(0x7fc00000);
-            }
+            // row scales; their maximum over the allowed rows feeds the accumulator bound, and a
+            // block with a negative or non-finite one (no encoder writes such) is always scored
+            const uint32_t slot = b * 32u + uint32_t(lane & 31);
+            bool ok = slot < a.n;
+            if (ok && a.mask != nullptr) ok = (uint32_t(a.mask[b >> 1] >> ((b & 1) * 32)) >> (lane & 31)) & 1u;
+            const float sc = ok ? a.scales[slot] : __int_as_float(0x7fc00000);
+            if (lane < 32) s_vs[wave * 32 + lane] = sc;
+            float vmax = ok ? sc : 0.0f;
+            bool odd = ok && !(sc >= 0.0f && sc < __int_as_float(0x7f800000));
+#pragma unroll
+            for (int d = 16; d >= 1; d >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, d));
+            odd_block = __any(odd);
+            inv_vmax = __builtin_amdgcn_readfirstlane(__float_as_int(1.0f / vmax));
         }
         if (!__syncthreads_or(has ? 1 : 0)) break;
+        TICK(0)
 
         // ---- tile phase ----
         // Scores of tile t for this wave's block; lane owns query t*32 + qn and rows
-        // 8*(r/4) + 4*h + r%4 (search.rs:1519-1524).  Candidates are rare, so one pass only
-        // tests the 16 scores and a second, entered by few waves, appends the ones that pass.
-        auto epilogue = [&](int t) {
-            const int q = t * kQTile + qn;
-            const float4 qp = *reinterpret_cast<const float4 *>(sq + q);
+        // 8*(r/4) + 4*h + r%4 (search.rs:1519-1524).  Entered only when some lane's largest
+        // accumulator reaches its query's bound, and then only the accumulators that reach it
+        // (one or two in the whole wave, as a rule) are scored and, if they pass, appended.
+        auto score_tile = [&](int q, int bound) {
+            const float4 qp = *reinterpret_cast<const float4 *>(&sq[q].qs);
             const float qs = qp.x, qb = qp.y, tau = qp.z;
-            const float4 *vs4 = reinterpret_cast<const float4 *>(s_vs + wave * 32 + 4 * h);
-            bool any = false;
+            const float *vs = s_vs + wave * 32 + 4 * h;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const float4 v = vs4[2 * g];
-                any |= fmaf(float(acc[4 * g + 0]), qs, qb) * v.x >= tau;
-                any |= fmaf(float(acc[4 * g + 1]), qs, qb) * v.y >= tau;
-                any |= fmaf(float(acc[4 * g + 2]), qs, qb) * v.z >= tau;
-                any |= fmaf(float(acc[4 * g + 3]), qs, qb) * v.w >= tau;
-            }
-            if (any) {
-                const float *vs = s_vs + wave * 32 + 4 * h;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
+            for (int r = 0; r < 16; ++r) {
+                if (acc[r] >= bound) {
                     const int i = 8 * (r >> 2) + (r & 3);
                     const float s = fmaf(float(acc[r]), qs, qb) * vs[i];
                     if (s >= tau) {
@@ -229,22 +259,42 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
                 }
             }
         };
-        for (int t = 0;; ++t) {
-            uint32_t b0 = 0;
-            if (t < nt) b0 = next_slice();
-            if (has && late && t > 0) epilogue(t - 1);
-            if (t == nt) break;
+        for (int t = 0; t < nt; ++t) {
+            const uint32_t b0 = slice_address();
+            int bound = 0;
+            const int q = t * kQTile + qn;
             if (has) {
                 acc = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                 slice_mfmas(IntC<0>{}, b0);
+                // the tile's accumulator bound, fetched and converted under the MFMAs
+                const float2 tq = *reinterpret_cast<const float2 *>(&sq[q].ta);
+                const float bf = fmaf(tq.x, __int_as_float(inv_vmax), -tq.y) - 1.0f;
+                asm("v_cvt_i32_f32 %0, %1" : "=v"(bound) : "v"(bf));   // saturates; NaN gives 0
+                if (odd_block) bound = int(0x80000000);
+            } else {
+                hand_over(IntC<kAhead - 2>{});
             }
-            const uint32_t b1 = next_slice();
+            TICK(5)
+            const uint32_t b1 = slice_address();
             if (has) {
                 slice_mfmas(IntC<1>{}, b1);
-                if (!late) epilogue(t);
+                TICK(5)
+                int m0 = max(max(acc[0], acc[1]), acc[2]), m1 = max(max(acc[3], acc[4]), acc[5]);
+                int m2 = max(max(acc[6], acc[7]), acc[8]), m3 = max(max(acc[9], acc[10]), acc[11]);
+                m0 = max(max(m0, acc[12]), acc[13]);
+                m1 = max(max(m1, acc[14]), acc[15]);
+                if (max(max(m0, m1), max(m2, m3)) >= bound) score_tile(q, bound);
+                TICK(7)
+            } else {
+                hand_over(IntC<kAhead - 2>{});
             }
         }
     }
+#ifdef WIDE_TIMING
+    if (blockIdx.x == 7 && lane == 0 && (wave == 0 || wave == 4) && step == 1)
+        printf("wave %d: block %llu vmwait %llu barrier %llu request %llu mfma %llu epi %llu\n", wave,
+               tk[0], tk[1], tk[2], tk[3], tk[5], tk[7]);
+#endif
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // requests still in flight write this workgroup's LDS
     __syncthreads();
     for (int q = tid; q < nq; q += kWideThreads) a.cand_cnt[size_t(q) * a.seg_stride + blockIdx.x] = sq[q].cnt;
@@ -313,7 +363,7 @@ int wide_min_queries(int nch) {
 
 static size_t wide_lds_bytes(int nch, int nq) {
     const size_t nq_pad = size_t((nq + kQTile - 1) / kQTile) * kQTile;
-    return size_t(kWideRing) * nch * 1024 + nq_pad * 16 + kWideWaves * 32 * 4 + 64;
+    return size_t(kWideRing) * nch * 1024 + nq_pad * sizeof(WideQuery) + kWideWaves * 32 * 4 + 64;
 }
 
 int wide_grid_blocks(int device) {
