@@ -102,12 +102,6 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
     const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
     const uint32_t step = a.b_step;
     const uint32_t nj = (a.n_blocks + step - 1) / step;
-#ifdef WIDE_TIMING
-    unsigned long long tk[8] = {0, 0, 0, 0, 0, 0, 0, 0}, t_last = __builtin_readcyclecounter();
-#define TICK(i) { const unsigned long long now_ = __builtin_readcyclecounter(); tk[i] += now_ - t_last; t_last = now_; }
-#else
-#define TICK(i)
-#endif
 
     // next live block of this workgroup (blocks m * gridDim.x + blockIdx.x), claimed wave by wave
     auto claim = [&]() -> uint32_t {
@@ -149,44 +143,46 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ys * (kPieces + 1)) : "memory");
         else
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ys * kPieces) : "memory");
-        TICK(1)
         __syncthreads();
-        TICK(2)
         request_next();
-        TICK(3)
     };
     // slices 0..3 requested, slice 0 whole: the state the first hand-over expects
     for (int i = 0; i < kAhead - 1; ++i) request_next();
     hand_over(IntC<kAhead - 2>{});
     int use_slot = 0;                                       // ring slot of the slice consumed next
-    auto slice_address = [&]() -> uint32_t {
-        const uint32_t bp = lds_b + uint32_t(use_slot) * kSlice + lane16;
-        use_slot = use_slot + 1 == kWideRing ? 0 : use_slot + 1;
-        return bp;
-    };
 
     v4i alo[NCH], ahi[NCH];
     v16i acc;
-    // The NCH MFMAs of one slice.  MFMA m takes chunk HALF * NCH/2 + m/2 (low nibbles for even m,
-    // high for odd) against the 1 KiB of weights at m * 1024, which come through NB registers
-    // requested NB MFMAs ahead; the hand-over of the next slice sits in the middle.
-    auto slice_mfmas = [&](auto half, uint32_t baddr) {
-        constexpr int c0 = decltype(half)::value * (NCH / 2);
-        v4i w[NB];
+    // B operands travel through NB registers requested NB MFMAs ahead, in one stream that runs on
+    // from a slice into the next (whole since the hand-over in the middle of the current one): a
+    // wave opens the stream at the start of a round of tiles and closes it at the end.
+    static_assert(NCH % NB == 0 && NB <= NCH / 2, "the operand ring must line up with the slices");
+    v4i w[NB];
+    auto open_stream = [&]() {
+        const uint32_t baddr = lds_b + uint32_t(use_slot) * kSlice + lane16;
         static_for<NB>([&](auto mm) { lds_read16_async<decltype(mm)::value * 1024>(w[decltype(mm)::value], baddr); });
+    };
+    auto close_stream = [&]() {    // the reads into the slice after the round's last are dropped, once landed
+        static_for<NB>([&](auto mm) { lds_wait<0>(w[decltype(mm)::value]); });
+    };
+    // The NCH MFMAs of one slice.  MFMA m takes chunk HALF * NCH/2 + m/2 (low nibbles for even m,
+    // high for odd) against the 1 KiB of weights at m * 1024; the hand-over of the next slice
+    // sits in the middle.
+    auto slice_mfmas = [&](auto half) {
+        constexpr int c0 = decltype(half)::value * (NCH / 2);
+        const uint32_t baddr = lds_b + uint32_t(use_slot) * kSlice + lane16;
+        use_slot = use_slot + 1 == kWideRing ? 0 : use_slot + 1;
+        const uint32_t naddr = lds_b + uint32_t(use_slot) * kSlice + lane16;
         static_for<NCH>([&](auto mm) {
             constexpr int m = decltype(mm)::value;
-            constexpr int younger = NCH - 1 - m < NB - 1 ? NCH - 1 - m : NB - 1;
-            if constexpr (m == NCH / 2) {
-                TICK(5)
-                hand_over(IntC<kAhead - 2>{});
-            }
-            lds_wait<younger>(w[m % NB]);
+            if constexpr (m == NCH / 2) hand_over(IntC<kAhead - 2>{});
+            lds_wait<NB - 1>(w[m % NB]);
             if constexpr ((m & 1) == 0)
                 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo[c0 + m / 2], w[m % NB], acc, 0, 0, 0);
             else
                 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi[c0 + m / 2], w[m % NB], acc, 0, 0, 0);
             if constexpr (m + NB < NCH) lds_read16_async<(m + NB) * 1024>(w[m % NB], baddr);
+            else lds_read16_async<(m + NB - NCH) * 1024>(w[m % NB], naddr);
         });
     };
 
@@ -234,7 +230,6 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
             inv_vmax = __builtin_amdgcn_readfirstlane(__float_as_int(1.0f / vmax));
         }
         if (!__syncthreads_or(has ? 1 : 0)) break;
-        TICK(0)
 
         // ---- tile phase ----
         // Scores of tile t for this wave's block; lane owns query t*32 + qn and rows
@@ -259,42 +254,32 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
                 }
             }
         };
+        if (has) open_stream();
         for (int t = 0; t < nt; ++t) {
-            const uint32_t b0 = slice_address();
             int bound = 0;
             const int q = t * kQTile + qn;
             if (has) {
                 acc = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                slice_mfmas(IntC<0>{}, b0);
+                slice_mfmas(IntC<0>{});
                 // the tile's accumulator bound, fetched and converted under the MFMAs
                 const float2 tq = *reinterpret_cast<const float2 *>(&sq[q].ta);
                 const float bf = fmaf(tq.x, __int_as_float(inv_vmax), -tq.y) - 1.0f;
                 asm("v_cvt_i32_f32 %0, %1" : "=v"(bound) : "v"(bf));   // saturates; NaN gives 0
                 if (odd_block) bound = int(0x80000000);
-            } else {
-                hand_over(IntC<kAhead - 2>{});
-            }
-            TICK(5)
-            const uint32_t b1 = slice_address();
-            if (has) {
-                slice_mfmas(IntC<1>{}, b1);
-                TICK(5)
+                slice_mfmas(IntC<1>{});
                 int m0 = max(max(acc[0], acc[1]), acc[2]), m1 = max(max(acc[3], acc[4]), acc[5]);
                 int m2 = max(max(acc[6], acc[7]), acc[8]), m3 = max(max(acc[9], acc[10]), acc[11]);
                 m0 = max(max(m0, acc[12]), acc[13]);
                 m1 = max(max(m1, acc[14]), acc[15]);
                 if (max(max(m0, m1), max(m2, m3)) >= bound) score_tile(q, bound);
-                TICK(7)
             } else {
+                use_slot = use_slot + 2 >= kWideRing ? use_slot + 2 - kWideRing : use_slot + 2;
+                hand_over(IntC<kAhead - 2>{});
                 hand_over(IntC<kAhead - 2>{});
             }
         }
+        if (has) close_stream();
     }
-#ifdef WIDE_TIMING
-    if (blockIdx.x == 7 && lane == 0 && (wave == 0 || wave == 4) && step == 1)
-        printf("wave %d: block %llu vmwait %llu barrier %llu request %llu mfma %llu epi %llu\n", wave,
-               tk[0], tk[1], tk[2], tk[3], tk[5], tk[7]);
-#endif
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // requests still in flight write this workgroup's LDS
     __syncthreads();
     for (int q = tid; q < nq; q += kWideThreads) a.cand_cnt[size_t(q) * a.seg_stride + blockIdx.x] = sq[q].cnt;
@@ -390,7 +375,7 @@ static hipError_t launch_wide_n(const ScanArgs &a, int grid, hipStream_t s) {
 // ceil(nq/32) weight tiles back to back, a.qscale / a.qbias / a.gtau indexed by query.
 hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s) {
     switch (a.nch) {
-        case 16: return launch_wide_n<16, 6>(a, grid, s);
+        case 16: return launch_wide_n<16, 4>(a, grid, s);
         case 20: return launch_wide_n<20, 4>(a, grid, s);
         case 24: return launch_wide_n<24, 2>(a, grid, s);
         default: return hipErrorInvalidValue;
