@@ -194,26 +194,24 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
         const bool has = j < nj;
         const uint32_t b = has ? j * step : 0u;
         if (has) {
-            // two bursts of NCH/2 chunks: the raw codes of a burst and the operands decoded so far
-            // have to fit the register file together
+            // the whole block in one burst: the previous block's operands are dead by now, so the
+            // raw codes (4 VGPRs per chunk) and the operands decoded from them so far (8 per chunk)
+            // fit the registers the operands alone need at the end
             const uint8_t *p = a.codes + size_t(b) * NCH * 1024;
-            static_for<2>([&](auto hh) {
-                constexpr int c0 = decltype(hh)::value * (NCH / 2);
-                u32x4 raw[NCH / 2];
-                static_for<NCH / 2>([&](auto cc) {
-                    constexpr int c = decltype(cc)::value;
-                    load16_async_s(raw[c], p + size_t(c0 + c) * 1024, lane16);
-                });
-                static_for<NCH / 2>([&](auto cc) {
-                    constexpr int c = decltype(cc)::value;
-                    wait_vm<NCH / 2 - 1 - c>(raw[c]);
-                    const uint32_t x[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
+            u32x4 raw[NCH];
+            static_for<NCH>([&](auto cc) {
+                constexpr int c = decltype(cc)::value;
+                load16_async_s(raw[c], p + size_t(c) * 1024, lane16);
+            });
+            static_for<NCH>([&](auto cc) {
+                constexpr int c = decltype(cc)::value;
+                wait_vm<NCH - 1 - c>(raw[c]);
+                const uint32_t x[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
 #pragma unroll
-                    for (int d = 0; d < 4; ++d) {
-                        alo[c0 + c][d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
-                        ahi[c0 + c][d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
-                    }
-                });
+                for (int d = 0; d < 4; ++d) {
+                    alo[c][d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
+                    ahi[c][d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
+                }
             });
             // row scales; their maximum over the allowed rows feeds the accumulator bound, and a
             // block with a negative or non-finite one (no encoder writes such) is always scored
