@@ -510,9 +510,10 @@ def test_all_equal_scores(T, oracle):
 
 
 # ---- batched permute-dot scan (more than 32 queries per launch) ----
-# dims 256/512/1536: weights of several tiles resident in LDS; 3072 and 2560: streamed in slices;
+# dims 256/512/1536: weights of several tiles resident in LDS (1536 with 97 queries: the wide
+# kernel, one pass for all); 3072 and 2560: streamed in slices;
 # 2624 (41 chunks, odd): no batched kernel applies, the single-tile scan serves the batch.
-@pytest.mark.parametrize("dim,n,nq", [(256, 40_003, 200), (1536, 20_011, 97), (512, 70_000, 129),
+@pytest.mark.parametrize("dim,n,nq", [(256, 40_003, 200), (1536, 20_011, 97), (1536, 9_001, 70), (512, 70_000, 129),
                                       (3072, 12_345, 131), (2560, 9_001, 70), (2624, 5_003, 40)])
 def test_batched_scan_matches_oracle(T, oracle, dim, n, nq):
     O = oracle

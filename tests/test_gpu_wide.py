@@ -23,10 +23,10 @@ def masks_for(T, n, seed):
     return [None if m is None else T.pack_mask(m)[0] for m in out]
 
 
-# dims 1536 and 1280 switch to the wide kernel at 256 queries, 1024 at 512; the query counts
+# dims 1536 and 1280 switch to the wide kernel at 97 queries, 1024 at 512; the query counts
 # leave a ragged last tile, and 1029 = one full chunk of 1024 plus a 5-query chunk that the
 # single-tile kernel serves
-@pytest.mark.parametrize("dim,n,nq", [(1536, 6_007, 300), (1280, 4_001, 257), (1024, 5_003, 520), (1536, 3_001, 1029)])
+@pytest.mark.parametrize("dim,n,nq", [(1536, 6_007, 300), (1280, 4_001, 257), (1280, 3_001, 100), (1024, 5_003, 520), (1536, 3_001, 1029)])
 def test_wide_scan_matches_oracle(T, oracle, dim, n, nq):
     oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=dim + n))
     q = unit_gaussian(nq, dim, seed=77)
@@ -34,7 +34,7 @@ def test_wide_scan_matches_oracle(T, oracle, dim, n, nq):
     for words in masks_for(T, n, 8):
         for k in (1, 10, 100):
             s, i = ix.search(q, k, mask_words=words)
-            assert ix.queries_per_launch() >= 256 or nq == 1029
+            assert ix.queries_per_launch() == nq or nq == 1029
             os_, oi = oidx.search(q, k, mask_words=words)
             assert np.array_equal(i, oi), k
             assert bits_equal(s, os_), k

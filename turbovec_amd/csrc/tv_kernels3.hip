@@ -336,10 +336,12 @@ hipError_t launch_probe_mfma(int device, int iters, uint32_t *sink, double *ops,
 }
 
 // Smallest chunk of queries the wide kernel is the faster one for (measured against the
-// tile-group kernels on 4-bit indexes of 1024, 1280 and 1536 dimensions); 0 = never.  Below
-// 1024 dimensions a tile is too few MFMAs for its two barriers and its epilogue.
+// tile-group kernels on 4-bit indexes of 1024, 1280 and 1536 dimensions); 0 = never.  At 1280
+// and 1536 dimensions that is as soon as the tile-group kernel would need a second pass over
+// the codes (it serves 96 queries per pass there).  Below 1024 dimensions a tile is too few
+// MFMAs for its two barriers and its epilogue.
 int wide_min_queries(int nch) {
-    if (nch == 24 || nch == 20) return 256;
+    if (nch == 24 || nch == 20) return 97;
     if (nch == 16) return 512;
     return 0;
 }
