@@ -61,18 +61,25 @@ struct WideQuery {
     float pad2;
 };
 
-template <int NCH, int NB>
-__global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
-    static_assert(NCH % 2 == 0, "a slice is half of the chunks");
+// WAVES = 8 (two per SIMD, 256 VGPRs each) holds rows of up to 24 chunks; WAVES = 4 (one per SIMD)
+// gives a wave the whole 512-register file -- the compiler keeps what does not fit the VGPRs in
+// AGPRs, which the MFMA reads as A operands directly -- for rows of up to 48 chunks.  A tile's
+// weights go through the ring in SPT slices of NCH / SPT chunks.
+template <int NCH, int NB, int WAVES, int SPT>
+__global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide(ScanArgs a) {
+    static_assert(NCH % SPT == 0, "a slice is a whole number of chunks");
     extern __shared__ __align__(16) uint8_t smem[];
-    constexpr int kSlice = NCH * 1024;                      // half a tile: NCH/2 chunks x (low, high) x 1 KiB
-    constexpr int kPieces = NCH / kWideWaves;               // direct-to-LDS loads per wave and slice ...
-    constexpr int kExtra = NCH % kWideWaves;                // ... plus one more in the first kExtra waves
+    constexpr int kWideThreads = WAVES * 64, kWideWaves = WAVES;
+    constexpr int kSC = NCH / SPT;                          // chunks per slice
+    constexpr int kM = 2 * kSC;                             // MFMAs per wave and slice: (low, high) of each chunk
+    constexpr int kSlice = kM * 1024;                       // bytes: one 1 KiB B operand per MFMA
+    constexpr int kPieces = kM / kWideWaves;                // direct-to-LDS loads per wave and slice ...
+    constexpr int kExtra = kM % kWideWaves;                 // ... plus one more in the first kExtra waves
     constexpr int kAhead = kWideRing - 1;
     const int nq = a.nq_tile;
     const int nt = (nq + kQTile - 1) / kQTile;
     const int nq_pad = nt * kQTile;
-    const int n_slices = 2 * nt;                            // per pass over the tiles; the host guarantees >= kAhead
+    const int n_slices = SPT * nt;                          // per pass over the tiles; the host guarantees >= kAhead
     WideQuery *sq = reinterpret_cast<WideQuery *>(smem + kWideRing * kSlice);
     float *s_vs = reinterpret_cast<float *>(sq + nq_pad);   // [waves][32]: row scales, NaN where not allowed
     uint32_t *snext = reinterpret_cast<uint32_t *>(s_vs + kWideWaves * 32);
@@ -116,7 +123,7 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
         }
     };
 
-    // The weights are one periodic stream of slices (slice s = half s & 1 of tile s >> 1, kSlice
+    // The weights are one periodic stream of slices (slice s = part s % SPT of tile s / SPT, kSlice
     // contiguous bytes; after the last tile the first follows again for the next round of blocks).
     // Stream position g lives in ring slot g % kWideRing.  Half way through the MFMAs of slice g
     // every wave waits for its own pieces of slice g + 1, meets the others at a barrier -- after
@@ -156,7 +163,7 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
     // B operands travel through NB registers requested NB MFMAs ahead, in one stream that runs on
     // from a slice into the next (whole since the hand-over in the middle of the current one): a
     // wave opens the stream at the start of a round of tiles and closes it at the end.
-    static_assert(NCH % NB == 0 && NB <= NCH / 2, "the operand ring must line up with the slices");
+    static_assert(kM % NB == 0 && NB <= kM / 2, "the operand ring must line up with the slices");
     v4i w[NB];
     auto open_stream = [&]() {
         const uint32_t baddr = lds_b + uint32_t(use_slot) * kSlice + lane16;
@@ -165,24 +172,24 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
     auto close_stream = [&]() {    // the reads into the slice after the round's last are dropped, once landed
         static_for<NB>([&](auto mm) { lds_wait<0>(w[decltype(mm)::value]); });
     };
-    // The NCH MFMAs of one slice.  MFMA m takes chunk HALF * NCH/2 + m/2 (low nibbles for even m,
+    // The kM MFMAs of one slice.  MFMA m takes chunk PART * kSC + m/2 (low nibbles for even m,
     // high for odd) against the 1 KiB of weights at m * 1024; the hand-over of the next slice
     // sits in the middle.
-    auto slice_mfmas = [&](auto half) {
-        constexpr int c0 = decltype(half)::value * (NCH / 2);
+    auto slice_mfmas = [&](auto part) {
+        constexpr int c0 = decltype(part)::value * kSC;
         const uint32_t baddr = lds_b + uint32_t(use_slot) * kSlice + lane16;
         use_slot = use_slot + 1 == kWideRing ? 0 : use_slot + 1;
         const uint32_t naddr = lds_b + uint32_t(use_slot) * kSlice + lane16;
-        static_for<NCH>([&](auto mm) {
+        static_for<kM>([&](auto mm) {
             constexpr int m = decltype(mm)::value;
-            if constexpr (m == NCH / 2) hand_over(IntC<kAhead - 2>{});
+            if constexpr (m == kM / 2) hand_over(IntC<kAhead - 2>{});
             lds_wait<NB - 1>(w[m % NB]);
             if constexpr ((m & 1) == 0)
                 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo[c0 + m / 2], w[m % NB], acc, 0, 0, 0);
             else
                 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi[c0 + m / 2], w[m % NB], acc, 0, 0, 0);
-            if constexpr (m + NB < NCH) lds_read16_async<(m + NB) * 1024>(w[m % NB], baddr);
-            else lds_read16_async<(m + NB - NCH) * 1024>(w[m % NB], naddr);
+            if constexpr (m + NB < kM) lds_read16_async<(m + NB) * 1024>(w[m % NB], baddr);
+            else lds_read16_async<(m + NB - kM) * 1024>(w[m % NB], naddr);
         });
     };
 
@@ -264,16 +271,16 @@ __global__ __launch_bounds__(kWideThreads, 2) void k_scan_p4_wide(ScanArgs a) {
                 const float bf = fmaf(tq.x, __int_as_float(inv_vmax), -tq.y) - 1.0f;
                 asm("v_cvt_i32_f32 %0, %1" : "=v"(bound) : "v"(bf));   // saturates; NaN gives 0
                 if (odd_block) bound = int(0x80000000);
-                slice_mfmas(IntC<1>{});
+                static_for<SPT - 1>([&](auto pp) { slice_mfmas(IntC<decltype(pp)::value + 1>{}); });
                 int m0 = max(max(acc[0], acc[1]), acc[2]), m1 = max(max(acc[3], acc[4]), acc[5]);
                 int m2 = max(max(acc[6], acc[7]), acc[8]), m3 = max(max(acc[9], acc[10]), acc[11]);
                 m0 = max(max(m0, acc[12]), acc[13]);
                 m1 = max(max(m1, acc[14]), acc[15]);
                 if (max(max(m0, m1), max(m2, m3)) >= bound) score_tile(q, bound);
             } else {
-                use_slot = use_slot + 2 >= kWideRing ? use_slot + 2 - kWideRing : use_slot + 2;
-                hand_over(IntC<kAhead - 2>{});
-                hand_over(IntC<kAhead - 2>{});
+                use_slot = (use_slot + SPT) % kWideRing;
+#pragma unroll
+                for (int i = 0; i < SPT; ++i) hand_over(IntC<kAhead - 2>{});
             }
         }
         if (has) close_stream();
@@ -342,13 +349,14 @@ hipError_t launch_probe_mfma(int device, int iters, uint32_t *sink, double *ops,
 // MFMAs for its two barriers and its epilogue.
 int wide_min_queries(int nch) {
     if (nch == 24 || nch == 20) return 97;
+    if (nch == 32 || nch == 40 || nch == 48) return 97;
     if (nch == 16) return 512;
     return 0;
 }
 
-static size_t wide_lds_bytes(int nch, int nq) {
+static size_t wide_lds_bytes(int slice_bytes, int nq) {
     const size_t nq_pad = size_t((nq + kQTile - 1) / kQTile) * kQTile;
-    return size_t(kWideRing) * nch * 1024 + nq_pad * sizeof(WideQuery) + kWideWaves * 32 * 4 + 64;
+    return size_t(kWideRing) * slice_bytes + nq_pad * sizeof(WideQuery) + kWideWaves * 32 * 4 + 64;
 }
 
 int wide_grid_blocks(int device) {
@@ -359,15 +367,15 @@ int wide_grid_blocks(int device) {
     return cus;      // one 8-wave workgroup per CU: its LDS holds the slice ring
 }
 
-template <int NCH, int NB>
+template <int NCH, int NB, int WAVES = 8, int SPT = 2>
 static hipError_t launch_wide_n(const ScanArgs &a, int grid, hipStream_t s) {
-    const size_t lds = wide_lds_bytes(NCH, a.nq_tile);
+    const size_t lds = wide_lds_bytes(2 * (NCH / SPT) * 1024, a.nq_tile);
     if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_p4_wide<NCH, NB>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_p4_wide<NCH, NB, WAVES, SPT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((k_scan_p4_wide<NCH, NB>), dim3(grid), dim3(kWideThreads), lds, s, a);
+    hipLaunchKernelGGL((k_scan_p4_wide<NCH, NB, WAVES, SPT>), dim3(grid), dim3(WAVES * 64), lds, s, a);
     return hipGetLastError();
 }
 
@@ -378,6 +386,9 @@ hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s) {
         case 16: return launch_wide_n<16, 4>(a, grid, s);
         case 20: return launch_wide_n<20, 4>(a, grid, s);
         case 24: return launch_wide_n<24, 2>(a, grid, s);
+        case 32: return launch_wide_n<32, 4, 4, 4>(a, grid, s);
+        case 40: return launch_wide_n<40, 4, 4, 4>(a, grid, s);
+        case 48: return launch_wide_n<48, 4, 4, 4>(a, grid, s);
         default: return hipErrorInvalidValue;
     }
 }
