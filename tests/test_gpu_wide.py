@@ -24,11 +24,13 @@ def masks_for(T, n, seed):
 
 
 # dims 1280 to 3072 switch to the wide kernel at 97 queries (2048 and up: its four-wave form, a
-# row's operands in 512 registers), 1024 at 512; the query counts
+# row's operands in 512 registers), dims up to 1024 at 129 (256 to 768: two to four blocks per wave); the query counts
 # leave a ragged last tile, and 1029 = one full chunk of 1024 plus a 5-query chunk that the
 # single-tile kernel serves
 @pytest.mark.parametrize("dim,n,nq", [(1536, 6_007, 300), (1280, 4_001, 257), (1280, 3_001, 100), (1024, 5_003, 520), (1536, 3_001, 1029),
-                                      (2048, 3_001, 200), (2560, 2_001, 100), (3072, 2_501, 260)])
+                                      (2048, 3_001, 200), (2560, 2_001, 100), (3072, 2_501, 260),
+                                      (256, 20_011, 333), (384, 9_001, 130), (512, 12_345, 200), (768, 7_003, 290),
+                                      (1024, 4_001, 129)])
 def test_wide_scan_matches_oracle(T, oracle, dim, n, nq):
     oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=dim + n))
     q = unit_gaussian(nq, dim, seed=77)
@@ -59,7 +61,8 @@ def test_wide_launch_covers_the_chunk(T, oracle):
 
 # device-encoded index too large for the oracle: the wide kernel against the tile-group
 # kernels and the exact full-list path on the same index (k up to the sort capacity's regime)
-@pytest.mark.parametrize("dim,n,nq", [(1536, 300_000, 1024 + 300), (1024, 200_000, 700), (3072, 150_000, 1024)])
+@pytest.mark.parametrize("dim,n,nq", [(1536, 300_000, 1024 + 300), (1024, 200_000, 700), (3072, 150_000, 1024),
+                                      (256, 500_000, 1024), (768, 400_000, 600)])
 def test_wide_scan_matches_other_paths(T, dim, n, nq):
     dev = torch.device("cuda:0")
     gen = torch.Generator(device=dev)

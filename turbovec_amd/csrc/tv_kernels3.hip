@@ -64,8 +64,10 @@ struct WideQuery {
 // WAVES = 8 (two per SIMD, 256 VGPRs each) holds rows of up to 24 chunks; WAVES = 4 (one per SIMD)
 // gives a wave the whole 512-register file -- the compiler keeps what does not fit the VGPRs in
 // AGPRs, which the MFMA reads as A operands directly -- for rows of up to 48 chunks.  A tile's
-// weights go through the ring in SPT slices of NCH / SPT chunks.
-template <int NCH, int NB, int WAVES, int SPT>
+// weights go through the ring in SPT slices of NCH / SPT chunks.  Short rows leave registers
+// for BLK blocks per wave: every B operand read from LDS then feeds BLK MFMAs, and a tile's
+// barriers and epilogue are shared by BLK times the work.
+template <int NCH, int NB, int WAVES, int SPT, int BLK>
 __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide(ScanArgs a) {
     static_assert(NCH % SPT == 0, "a slice is a whole number of chunks");
     extern __shared__ __align__(16) uint8_t smem[];
@@ -81,8 +83,8 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     const int nq_pad = nt * kQTile;
     const int n_slices = SPT * nt;                          // per pass over the tiles; the host guarantees >= kAhead
     WideQuery *sq = reinterpret_cast<WideQuery *>(smem + kWideRing * kSlice);
-    float *s_vs = reinterpret_cast<float *>(sq + nq_pad);   // [waves][32]: row scales, NaN where not allowed
-    uint32_t *snext = reinterpret_cast<uint32_t *>(s_vs + kWideWaves * 32);
+    float *s_vs = reinterpret_cast<float *>(sq + nq_pad);   // [waves][BLK][32]: row scales, NaN where not allowed
+    uint32_t *snext = reinterpret_cast<uint32_t *>(s_vs + kWideWaves * BLK * 32);
     const uint32_t lds_b = uint32_t(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)smem));
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -158,8 +160,8 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     hand_over(IntC<kAhead - 2>{});
     int use_slot = 0;                                       // ring slot of the slice consumed next
 
-    v4i alo[NCH], ahi[NCH];
-    v16i acc;
+    v4i alo[BLK][NCH], ahi[BLK][NCH];
+    v16i acc[BLK];
     // B operands travel through NB registers requested NB MFMAs ahead, in one stream that runs on
     // from a slice into the next (whole since the hand-over in the middle of the current one): a
     // wave opens the stream at the start of a round of tiles and closes it at the end.
@@ -184,99 +186,121 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
             constexpr int m = decltype(mm)::value;
             if constexpr (m == kM / 2) hand_over(IntC<kAhead - 2>{});
             lds_wait<NB - 1>(w[m % NB]);
-            if constexpr ((m & 1) == 0)
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo[c0 + m / 2], w[m % NB], acc, 0, 0, 0);
-            else
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi[c0 + m / 2], w[m % NB], acc, 0, 0, 0);
+            static_for<BLK>([&](auto kk) {
+                constexpr int k = decltype(kk)::value;
+                if constexpr ((m & 1) == 0)
+                    acc[k] = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo[k][c0 + m / 2], w[m % NB], acc[k], 0, 0, 0);
+                else
+                    acc[k] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi[k][c0 + m / 2], w[m % NB], acc[k], 0, 0, 0);
+            });
             if constexpr (m + NB < kM) lds_read16_async<(m + NB) * 1024>(w[m % NB], baddr);
             else lds_read16_async<(m + NB - kM) * 1024>(w[m % NB], naddr);
         });
     };
 
-    int inv_vmax = 0;        // bits of 1 / (largest allowed row scale of the block); +inf when that is 0
-    bool odd_block = false;
+    int inv_vmax[BLK];       // bits of 1 / (largest allowed row scale of the block); +inf when that is 0
+    bool odd_block[BLK];
+    uint32_t blk[BLK];       // the wave's blocks of this round
     for (;;) {
         // ---- block phase: claim, load, decode into registers ----
-        const uint32_t j = claim();
-        const bool has = j < nj;
-        const uint32_t b = has ? j * step : 0u;
-        if (has) {
-            // the whole block in one burst: the previous block's operands are dead by now, so the
-            // raw codes (4 VGPRs per chunk) and the operands decoded from them so far (8 per chunk)
-            // fit the registers the operands alone need at the end
-            const uint8_t *p = a.codes + size_t(b) * NCH * 1024;
-            u32x4 raw[NCH];
-            static_for<NCH>([&](auto cc) {
-                constexpr int c = decltype(cc)::value;
-                load16_async_s(raw[c], p + size_t(c) * 1024, lane16);
-            });
-            static_for<NCH>([&](auto cc) {
-                constexpr int c = decltype(cc)::value;
-                wait_vm<NCH - 1 - c>(raw[c]);
-                const uint32_t x[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
+        bool has = false;
+        static_for<BLK>([&](auto kk) {
+            constexpr int k = decltype(kk)::value;
+            const uint32_t j = claim();
+            const bool has_k = j < nj;
+            has = has || has_k;
+            const uint32_t b = has_k ? j * step : 0u;
+            blk[k] = b;
+            float sc = __int_as_float(0x7fc00000);
+            bool ok = false;
+            if (has_k) {
+                // the whole block in one burst: the previous block's operands are dead by now, so
+                // the raw codes (4 VGPRs per chunk) and the operands decoded from them so far (8 per
+                // chunk) fit the registers the operands alone need at the end
+                const uint8_t *p = a.codes + size_t(b) * NCH * 1024;
+                u32x4 raw[NCH];
+                static_for<NCH>([&](auto cc) {
+                    constexpr int c = decltype(cc)::value;
+                    load16_async_s(raw[c], p + size_t(c) * 1024, lane16);
+                });
+                static_for<NCH>([&](auto cc) {
+                    constexpr int c = decltype(cc)::value;
+                    wait_vm<NCH - 1 - c>(raw[c]);
+                    const uint32_t x[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
 #pragma unroll
-                for (int d = 0; d < 4; ++d) {
-                    alo[c][d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
-                    ahi[c][d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
-                }
-            });
-            // row scales; their maximum over the allowed rows feeds the accumulator bound, and a
-            // block with a negative or non-finite one (no encoder writes such) is always scored
-            const uint32_t slot = b * 32u + uint32_t(lane & 31);
-            bool ok = slot < a.n;
-            if (ok && a.mask != nullptr) ok = (uint32_t(a.mask[b >> 1] >> ((b & 1) * 32)) >> (lane & 31)) & 1u;
-            const float sc = ok ? a.scales[slot] : __int_as_float(0x7fc00000);
-            if (lane < 32) s_vs[wave * 32 + lane] = sc;
+                    for (int d = 0; d < 4; ++d) {
+                        alo[k][c][d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
+                        ahi[k][c][d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
+                    }
+                });
+                const uint32_t slot = b * 32u + uint32_t(lane & 31);
+                ok = slot < a.n;
+                if (ok && a.mask != nullptr) ok = (uint32_t(a.mask[b >> 1] >> ((b & 1) * 32)) >> (lane & 31)) & 1u;
+                if (ok) sc = a.scales[slot];
+            }
+            // row scales (NaN where not allowed, and for a block slot left empty: its stale
+            // operands then score nothing); their maximum over the allowed rows feeds the
+            // accumulator bound, and a block with a negative or non-finite one (no encoder
+            // writes such) is always scored
+            if (lane < 32) s_vs[(wave * BLK + k) * 32 + lane] = sc;
             float vmax = ok ? sc : 0.0f;
-            bool odd = ok && !(sc >= 0.0f && sc < __int_as_float(0x7f800000));
+            const bool odd = ok && !(sc >= 0.0f && sc < __int_as_float(0x7f800000));
 #pragma unroll
             for (int d = 16; d >= 1; d >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, d));
-            odd_block = __any(odd);
-            inv_vmax = __builtin_amdgcn_readfirstlane(__float_as_int(1.0f / vmax));
-        }
+            odd_block[k] = __any(odd);
+            inv_vmax[k] = __builtin_amdgcn_readfirstlane(__float_as_int(1.0f / vmax));
+        });
         if (!__syncthreads_or(has ? 1 : 0)) break;
 
         // ---- tile phase ----
-        // Scores of tile t for this wave's block; lane owns query t*32 + qn and rows
+        // Scores of tile t for block k of this wave; lane owns query t*32 + qn and rows
         // 8*(r/4) + 4*h + r%4 (search.rs:1519-1524).  Entered only when some lane's largest
         // accumulator reaches its query's bound, and then only the accumulators that reach it
         // (one or two in the whole wave, as a rule) are scored and, if they pass, appended.
-        auto score_tile = [&](int q, int bound) {
+        auto score_tile = [&](int q, int bound, auto kk) {
+            constexpr int k = decltype(kk)::value;
             const float4 qp = *reinterpret_cast<const float4 *>(&sq[q].qs);
             const float qs = qp.x, qb = qp.y, tau = qp.z;
-            const float *vs = s_vs + wave * 32 + 4 * h;
+            const float *vs = s_vs + (wave * BLK + k) * 32 + 4 * h;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                if (acc[r] >= bound) {
+                if (acc[k][r] >= bound) {
                     const int i = 8 * (r >> 2) + (r & 3);
-                    const float s = fmaf(float(acc[r]), qs, qb) * vs[i];
+                    const float s = fmaf(float(acc[k][r]), qs, qb) * vs[i];
                     if (s >= tau) {
                         const uint32_t pos = atomicAdd(&sq[q].cnt, 1u);
                         if (pos < kSegCap)
                             a.cand[(size_t(q) * a.seg_stride + blockIdx.x) * kSegCap + pos] =
-                                sort_key(s, b * 32u + uint32_t(i + 4 * h));
+                                sort_key(s, blk[k] * 32u + uint32_t(i + 4 * h));
                     }
                 }
             }
         };
         if (has) open_stream();
         for (int t = 0; t < nt; ++t) {
-            int bound = 0;
             const int q = t * kQTile + qn;
             if (has) {
-                acc = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                static_for<BLK>([&](auto kk) { acc[decltype(kk)::value] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}; });
                 slice_mfmas(IntC<0>{});
-                // the tile's accumulator bound, fetched and converted under the MFMAs
+                // the tile's accumulator bounds, fetched and converted under the MFMAs
                 const float2 tq = *reinterpret_cast<const float2 *>(&sq[q].ta);
-                const float bf = fmaf(tq.x, __int_as_float(inv_vmax), -tq.y) - 1.0f;
-                asm("v_cvt_i32_f32 %0, %1" : "=v"(bound) : "v"(bf));   // saturates; NaN gives 0
-                if (odd_block) bound = int(0x80000000);
+                int bound[BLK];
+                static_for<BLK>([&](auto kk) {
+                    constexpr int k = decltype(kk)::value;
+                    const float bf = fmaf(tq.x, __int_as_float(inv_vmax[k]), -tq.y) - 1.0f;
+                    asm("v_cvt_i32_f32 %0, %1" : "=v"(bound[k]) : "v"(bf));   // saturates; NaN gives 0
+                    if (odd_block[k]) bound[k] = int(0x80000000);
+                });
                 static_for<SPT - 1>([&](auto pp) { slice_mfmas(IntC<decltype(pp)::value + 1>{}); });
-                int m0 = max(max(acc[0], acc[1]), acc[2]), m1 = max(max(acc[3], acc[4]), acc[5]);
-                int m2 = max(max(acc[6], acc[7]), acc[8]), m3 = max(max(acc[9], acc[10]), acc[11]);
-                m0 = max(max(m0, acc[12]), acc[13]);
-                m1 = max(max(m1, acc[14]), acc[15]);
-                if (max(max(m0, m1), max(m2, m3)) >= bound) score_tile(q, bound);
+                static_for<BLK>([&](auto kk) {
+                    constexpr int k = decltype(kk)::value;
+                    const v16i &c = acc[k];
+                    int m0 = max(max(c[0], c[1]), c[2]), m1 = max(max(c[3], c[4]), c[5]);
+                    int m2 = max(max(c[6], c[7]), c[8]), m3 = max(max(c[9], c[10]), c[11]);
+                    m0 = max(max(m0, c[12]), c[13]);
+                    m1 = max(max(m1, c[14]), c[15]);
+                    if (max(max(m0, m1), max(m2, m3)) >= bound[k]) score_tile(q, bound[k], kk);
+                });
             } else {
                 use_slot = (use_slot + SPT) % kWideRing;
 #pragma unroll
@@ -342,21 +366,24 @@ hipError_t launch_probe_mfma(int device, int iters, uint32_t *sink, double *ops,
     return hipGetLastError();
 }
 
-// Smallest chunk of queries the wide kernel is the faster one for (measured against the
-// tile-group kernels on 4-bit indexes of 1024, 1280 and 1536 dimensions); 0 = never.  At 1280
-// and 1536 dimensions that is as soon as the tile-group kernel would need a second pass over
-// the codes (it serves 96 queries per pass there).  Below 1024 dimensions a tile is too few
-// MFMAs for its two barriers and its epilogue.
+// Smallest chunk of queries the wide kernel is the faster one for; 0 = no instance for this row
+// length.  Measured against the tile-group kernels on 4-bit indexes of 256 to 3072 dimensions:
+// the wide kernel wins as soon as the tile-group kernel would need a second pass over the codes
+// (it serves 128 queries per pass up to 1024 dimensions, 96 at 1280 and 1536), by 1.4 to 1.6
+// times at 1024 queries; from 2048 dimensions, where the tile-group kernel streams its weights
+// too, it is level at 128 queries and 1.6 to 1.7 times faster at 1024.
 int wide_min_queries(int nch) {
-    if (nch == 24 || nch == 20) return 97;
-    if (nch == 32 || nch == 40 || nch == 48) return 97;
-    if (nch == 16) return 512;
-    return 0;
+    switch (nch) {
+        case 4: case 6: case 8: case 12: case 16: return 129;
+        case 20: case 24: return 97;
+        case 32: case 40: case 48: return 97;
+        default: return 0;
+    }
 }
 
-static size_t wide_lds_bytes(int slice_bytes, int nq) {
+static size_t wide_lds_bytes(int slice_bytes, int nq, int blk) {
     const size_t nq_pad = size_t((nq + kQTile - 1) / kQTile) * kQTile;
-    return size_t(kWideRing) * slice_bytes + nq_pad * sizeof(WideQuery) + kWideWaves * 32 * 4 + 64;
+    return size_t(kWideRing) * slice_bytes + nq_pad * sizeof(WideQuery) + size_t(kWideWaves) * blk * 32 * 4 + 64;
 }
 
 int wide_grid_blocks(int device) {
@@ -367,15 +394,15 @@ int wide_grid_blocks(int device) {
     return cus;      // one 8-wave workgroup per CU: its LDS holds the slice ring
 }
 
-template <int NCH, int NB, int WAVES = 8, int SPT = 2>
+template <int NCH, int NB, int WAVES = 8, int SPT = 2, int BLK = 1>
 static hipError_t launch_wide_n(const ScanArgs &a, int grid, hipStream_t s) {
-    const size_t lds = wide_lds_bytes(2 * (NCH / SPT) * 1024, a.nq_tile);
+    const size_t lds = wide_lds_bytes(2 * (NCH / SPT) * 1024, a.nq_tile, BLK);
     if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_p4_wide<NCH, NB, WAVES, SPT>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((k_scan_p4_wide<NCH, NB, WAVES, SPT>), dim3(grid), dim3(WAVES * 64), lds, s, a);
+    hipLaunchKernelGGL((k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK>), dim3(grid), dim3(WAVES * 64), lds, s, a);
     return hipGetLastError();
 }
 
@@ -383,6 +410,10 @@ static hipError_t launch_wide_n(const ScanArgs &a, int grid, hipStream_t s) {
 // ceil(nq/32) weight tiles back to back, a.qscale / a.qbias / a.gtau indexed by query.
 hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s) {
     switch (a.nch) {
+        case 4: return launch_wide_n<4, 2, 8, 1, 4>(a, grid, s);
+        case 6: return launch_wide_n<6, 2, 8, 1, 3>(a, grid, s);
+        case 8: return launch_wide_n<8, 4, 8, 1, 2>(a, grid, s);
+        case 12: return launch_wide_n<12, 2, 8, 2, 2>(a, grid, s);
         case 16: return launch_wide_n<16, 4>(a, grid, s);
         case 20: return launch_wide_n<20, 4>(a, grid, s);
         case 24: return launch_wide_n<24, 2>(a, grid, s);
