@@ -53,6 +53,15 @@ int ensure_workspace(tv_index *ix, size_t bytes) {
     return TV_OK;
 }
 
+int ensure_io(tv_index *ix, size_t bytes) {
+    if (bytes <= ix->io_bytes) return TV_OK;
+    if (ix->io) { TV_HIP(hipFree(ix->io)); ix->io = nullptr; ix->io_bytes = 0; }
+    bytes = round_up(bytes + bytes / 4, size_t(1) << 16);
+    TV_HIP(hipMalloc(&ix->io, bytes));
+    ix->io_bytes = bytes;
+    return TV_OK;
+}
+
 int ensure_capacity(tv_index *ix, size_t n_vectors) {
     const size_t blocks = (n_vectors + tv::kVecBlock - 1) / tv::kVecBlock;
     if (blocks <= ix->cap_blocks) return TV_OK;
@@ -523,7 +532,7 @@ int tv_index_destroy(tv_index *ix) {
     (void)hipSetDevice(ix->device);
     if (ix->stream) (void)hipStreamSynchronize(ix->stream);
     void *ptrs[] = {ix->d_signs, ix->d_perms, ix->d_centroids, ix->d_tq_shift, ix->d_tq_scale,
-                    ix->d_codes, ix->d_scales, ix->ws, ix->d_tau_open};
+                    ix->d_codes, ix->d_scales, ix->ws, ix->io, ix->d_tau_open};
     for (void *p : ptrs) if (p) (void)hipFree(p);
     if (ix->stream) (void)hipStreamDestroy(ix->stream);
     delete ix;
@@ -856,42 +865,33 @@ int tv_search(tv_index *ix, const float *queries, size_t nq, size_t k, const uin
     ix->last_scan_ms = 0.0f;
     ix->last_scan_launches = 0;
     if (k_eff == 0 || nq == 0) return TV_OK;
-    // host staging: queries, mask and results live in their own allocations so
-    // the per-chunk workspace can be re-carved freely
+    // host staging: queries, mask and results live in the index's own staging allocation (kept
+    // between calls, so a search allocates nothing once it has seen its largest batch), apart
+    // from the per-chunk workspace, which is re-carved freely
     const size_t dim = size_t(ix->geo.dim);
-    float *d_q = nullptr, *d_s = nullptr;
-    int64_t *d_i = nullptr;
-    uint64_t *d_m = nullptr;
-    int rc = TV_OK;
-    do {
-        if (hipMalloc(reinterpret_cast<void **>(&d_q), nq * dim * sizeof(float)) != hipSuccess ||
-            hipMalloc(reinterpret_cast<void **>(&d_s), nq * k_eff * sizeof(float)) != hipSuccess ||
-            hipMalloc(reinterpret_cast<void **>(&d_i), nq * k_eff * sizeof(int64_t)) != hipSuccess ||
-            (mask_words && hipMalloc(reinterpret_cast<void **>(&d_m), n_mask_words * 8) != hipSuccess)) {
-            g_last_error = "device allocation failed";
-            rc = TV_ERR_HIP;
-            break;
-        }
-        if (hipMemcpyAsync(d_q, queries, nq * dim * sizeof(float), hipMemcpyHostToDevice, ix->stream) != hipSuccess ||
-            (mask_words && hipMemcpyAsync(d_m, mask_words, n_mask_words * 8, hipMemcpyHostToDevice, ix->stream) != hipSuccess)) {
-            g_last_error = "host to device copy failed";
-            rc = TV_ERR_HIP;
-            break;
-        }
-        rc = search_device(ix, d_q, nq, k, d_m, n_allowed, d_s, d_i, nullptr);
-        if (rc != TV_OK) break;
-        if (hipMemcpyAsync(out_scores, d_s, nq * k_eff * sizeof(float), hipMemcpyDeviceToHost, ix->stream) != hipSuccess ||
-            hipMemcpyAsync(out_indices, d_i, nq * k_eff * sizeof(int64_t), hipMemcpyDeviceToHost, ix->stream) != hipSuccess ||
-            hipStreamSynchronize(ix->stream) != hipSuccess) {
-            g_last_error = "device to host copy failed";
-            rc = TV_ERR_HIP;
-        }
-    } while (0);
-    if (d_q) (void)hipFree(d_q);
-    if (d_s) (void)hipFree(d_s);
-    if (d_i) (void)hipFree(d_i);
-    if (d_m) (void)hipFree(d_m);
-    return rc;
+    const size_t q_bytes = round_up(nq * dim * sizeof(float), 256), s_bytes = round_up(nq * k_eff * sizeof(float), 256);
+    const size_t i_bytes = round_up(nq * k_eff * sizeof(int64_t), 256), m_bytes = mask_words ? round_up(n_mask_words * 8, 256) : 0;
+    int rc = ensure_io(ix, q_bytes + s_bytes + i_bytes + m_bytes);
+    if (rc != TV_OK) return rc;
+    uint8_t *base = static_cast<uint8_t *>(ix->io);
+    float *d_q = reinterpret_cast<float *>(base);
+    float *d_s = reinterpret_cast<float *>(base + q_bytes);
+    int64_t *d_i = reinterpret_cast<int64_t *>(base + q_bytes + s_bytes);
+    uint64_t *d_m = mask_words ? reinterpret_cast<uint64_t *>(base + q_bytes + s_bytes + i_bytes) : nullptr;
+    if (hipMemcpyAsync(d_q, queries, nq * dim * sizeof(float), hipMemcpyHostToDevice, ix->stream) != hipSuccess ||
+        (mask_words && hipMemcpyAsync(d_m, mask_words, n_mask_words * 8, hipMemcpyHostToDevice, ix->stream) != hipSuccess)) {
+        g_last_error = "host to device copy failed";
+        return TV_ERR_HIP;
+    }
+    rc = search_device(ix, d_q, nq, k, d_m, n_allowed, d_s, d_i, nullptr);
+    if (rc != TV_OK) return rc;
+    if (hipMemcpyAsync(out_scores, d_s, nq * k_eff * sizeof(float), hipMemcpyDeviceToHost, ix->stream) != hipSuccess ||
+        hipMemcpyAsync(out_indices, d_i, nq * k_eff * sizeof(int64_t), hipMemcpyDeviceToHost, ix->stream) != hipSuccess ||
+        hipStreamSynchronize(ix->stream) != hipSuccess) {
+        g_last_error = "device to host copy failed";
+        return TV_ERR_HIP;
+    }
+    return TV_OK;
 }
 
 int tv_debug_scan(tv_index *ix, const float *queries, size_t nq, int32_t *acc_out, float *scores_out) {

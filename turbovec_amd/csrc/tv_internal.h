@@ -160,6 +160,8 @@ struct tv_index {
     // per-search workspace, grown on demand, guarded by mu
     mutable std::mutex mu;
     void *ws = nullptr;
+    void *io = nullptr;            // staging for tv_search's host buffers (queries, mask, results); grows, never shrinks
+    size_t io_bytes = 0;
     size_t ws_bytes = 0;
     float last_scan_ms = 0.0f;
     int last_scan_launches = 0;
