@@ -86,3 +86,34 @@ def test_wide_scan_matches_other_paths(T, dim, n, nq):
         s, i = ix.search(q, 10, mask_words=words)
         assert np.array_equal(i[:40], i3) and bits_equal(s[:40], s3)
     ix.close()
+
+
+def test_wide_scan_with_wild_row_scales(T, oracle):
+    """Row scales far from the encoder's (zeros, tiny, huge: the accumulator bound divides by the
+    block's largest one) against the oracle; with negative ones mixed in (a foreign snapshot
+    could hold them; such blocks skip the bound) against the tile-group and exact paths."""
+    dim, n, nq = 1536, 5_003, 200
+    oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=31))
+    rng = np.random.default_rng(32)
+    factors = rng.choice(np.array([0.0, 1e-12, 1e-3, 1.0, 3.7, 1e6], np.float32), size=n)
+    oidx.scales = (oidx.scales * factors).astype(np.float32)
+    q = unit_gaussian(nq, dim, seed=33)
+    ix = to_native(T, oidx)
+    for k in (1, 10, 100):
+        s, i = ix.search(q, k)
+        assert ix.queries_per_launch() == nq
+        os_, oi = oidx.search(q, k)
+        assert np.array_equal(i, oi) and bits_equal(s, os_), k
+    ix.close()
+    oidx.scales[rng.random(n) < 0.02] *= np.float32(-1.0)
+    ix = to_native(T, oidx)
+    for k in (10, 100):
+        s, i = ix.search(q, k)
+        ix.set_path(4)
+        s2, i2 = ix.search(q, k)
+        ix.set_path(1)
+        s3, i3 = ix.search(q, k)
+        ix.set_path(0)
+        assert np.array_equal(i, i2) and bits_equal(s, s2), k
+        assert np.array_equal(i, i3) and bits_equal(s, s3), k
+    ix.close()
