@@ -10,6 +10,9 @@
 //     gather: (x[perm0[i]] * inv) * sign0[i];
 //   * the reconstruction inner product runs in 4 interleaved f64 chains
 //     (element j feeds chain j % 4), folded pairwise; 4 lanes carry them.
+// Only the additions of those chains are sequential: the squares and the f64
+// products they add up are computed by all threads first, each by the same
+// operations as in the reference, and parked in LDS.
 #include <hip/hip_runtime.h>
 
 #include "tv_internal.h"
@@ -65,12 +68,11 @@ __global__ __launch_bounds__(256) void k_encode(EncodeArgs a) {
     __syncthreads();
 
     // encode.rs:920-932: c[j % 8] += x * x (separate multiply and add), then the pairwise fold
+    for (int i = t; i < dim; i += 256) B[i] = A[i] * A[i];
+    __syncthreads();
     if (t < 8) {
         float c = 0.0f;
-        for (int j = t; j < dim; j += 8) {
-            const float sq = A[j] * A[j];
-            c = c + sq;
-        }
+        for (int j = t; j < dim; j += 8) c = c + B[j];
         red[t] = c;
     }
     __syncthreads();
@@ -105,16 +107,18 @@ __global__ __launch_bounds__(256) void k_encode(EncodeArgs a) {
     __syncthreads();
 
     // encode.rs:1442-1475: inner = <rotated, reconstruction> in f64, four chains by j % 4
+    double *terms = reinterpret_cast<double *>(enc_lds + 2 * dim);
+    for (int j = t; j < dim; j += 256) {
+        const float sh = a.shift ? a.shift[j] : 0.0f;
+        const float sc = a.scale ? a.scale[j] : 1.0f;
+        const float inv_sc = 1.0f / sc;                       // encode.rs:594
+        const double recon = double(s_cen[codes[j]]) * double(inv_sc) - double(sh);
+        terms[j] = double(B[j]) * recon;
+    }
+    __syncthreads();
     if (t < 4) {
         double ch = 0.0;
-        for (int j = t; j < dim; j += 4) {
-            const float sh = a.shift ? a.shift[j] : 0.0f;
-            const float sc = a.scale ? a.scale[j] : 1.0f;
-            const float inv_sc = 1.0f / sc;                   // encode.rs:594
-            const double recon = double(s_cen[codes[j]]) * double(inv_sc) - double(sh);
-            const double term = double(B[j]) * recon;
-            ch = ch + term;
-        }
+        for (int j = t; j < dim; j += 4) ch = ch + terms[j];
         dred[t] = ch;
     }
     __syncthreads();
@@ -148,7 +152,7 @@ hipError_t launch_encode(const float *d_vecs, size_t n_new, size_t old_n, const 
     a.inv_sqrt_block = inv_sqrt_block;
     a.nat = d_native; a.scales = d_scales; a.old_n = old_n; a.n_new = n_new;
     a.rot_out = d_rot_out;
-    const size_t lds = size_t(2) * g.dim * sizeof(float);
+    const size_t lds = size_t(2) * g.dim * sizeof(float) + size_t(g.dim) * sizeof(double);   // A, B, f64 terms
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_encode),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
