@@ -920,6 +920,7 @@ __global__ __launch_bounds__(256) void k_merge(const float *__restrict__ part_sc
 // ===========================================================================
 
 constexpr int kFinalThreads = 1024;
+constexpr int kFinalLong = kFinalCap / 4;   // segments of more than 4 keys that fit the sort buffer
 
 __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restrict__ cand,
                                                const uint32_t *__restrict__ cand_cnt, uint32_t n_seg,
@@ -929,12 +930,13 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
                                                int tau_stride_q) {
     __shared__ uint64_t keys[kFinalCap];
     __shared__ uint32_t wave_sum[kFinalThreads / 64];
-    __shared__ uint32_t any_full;
+    __shared__ uint32_t any_full, long_n;
+    __shared__ uint32_t long_seg[kFinalLong], long_pos[kFinalLong];
     const int qn = blockIdx.x;
     const int t = threadIdx.x;
     const bool sampling = tau_out != nullptr;
     int *tau_slot = sampling ? tau_out + (qn / tau_stride_q) * kQTile + qn % tau_stride_q : nullptr;
-    if (t == 0) any_full = 0u;
+    if (t == 0) { any_full = 0u; long_n = 0u; }
     __syncthreads();
     // every thread owns a contiguous run of this query's segments
     const uint32_t per = (n_seg + kFinalThreads - 1) / kFinalThreads;
@@ -966,30 +968,106 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
         if (t == 0) *tau_slot = kTauInit;  // too few allowed slots sampled: the floor stays open
         return;
     }
-    // gather (a sampling level may keep any subset: dropping what does not fit only loosens the floor)
+    // gather (a sampling level may keep any subset: dropping what does not fit only loosens the floor).
+    // A thread copies a short segment itself, its loads in flight together; long ones (the first
+    // sampling level fills a few segments to the brim) go on a list the waves then share, a
+    // segment per wave and turn, a key per lane.
     uint32_t pos = base;
     for (uint32_t sg = s0; sg < s1; ++sg) {
         const uint32_t c = min(cnt[sg], uint32_t(kSegCap));
         const uint64_t *src = cand + (size_t(qn) * seg_stride + sg) * kSegCap;
-        for (uint32_t e = 0; e < c; ++e, ++pos)
-            if (pos < uint32_t(kFinalCap)) keys[pos] = src[e];
+        if (c <= 4) {
+            uint64_t v[4];
+#pragma unroll
+            for (uint32_t e = 0; e < 4; ++e) v[e] = e < c ? src[e] : 0ull;
+#pragma unroll
+            for (uint32_t e = 0; e < 4; ++e)
+                if (e < c && pos + e < uint32_t(kFinalCap)) keys[pos + e] = v[e];
+        } else {
+            const uint32_t slot = atomicAdd(&long_n, 1u);
+            if (slot < uint32_t(kFinalLong)) {
+                long_seg[slot] = sg;
+                long_pos[slot] = pos;
+            } else {                      // more long segments than the list holds: copy in place
+                for (uint32_t e = 0; e < c; ++e)
+                    if (pos + e < uint32_t(kFinalCap)) keys[pos + e] = src[e];
+            }
+        }
+        pos += c;
+    }
+    __syncthreads();
+    const uint32_t n_long = min(long_n, uint32_t(kFinalLong));
+    for (uint32_t i = uint32_t(t >> 6); i < n_long; i += kFinalThreads / 64) {
+        const uint32_t sg = long_seg[i], at = long_pos[i] + uint32_t(t & 63);
+        const uint32_t c = min(cnt[sg], uint32_t(kSegCap));
+        if (uint32_t(t & 63) < c && at < uint32_t(kFinalCap))
+            keys[at] = cand[(size_t(qn) * seg_stride + sg) * kSegCap + (t & 63)];
     }
     const uint32_t c_all = min(total, uint32_t(kFinalCap));
-    uint32_t sort_n = 2;
+    const uint32_t need = sampling ? min(uint32_t(k_floor), c_all) : uint32_t(k_eff);   // leading keys wanted, in order
+    uint32_t sort_n = need <= 64u ? 64u : 2u;
     while (sort_n < c_all) sort_n <<= 1;
     __syncthreads();
     for (uint32_t i = c_all + t; i < sort_n; i += kFinalThreads) keys[i] = 0ull;
     __syncthreads();
-    for (uint32_t size = 2; size <= sort_n; size <<= 1) {
-        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
-            for (uint32_t i = t; i < sort_n / 2; i += kFinalThreads) {
-                const uint32_t lo = 2 * i - (i & (stride - 1));
-                const uint32_t hi = lo + stride;
-                const bool desc = (lo & size) == 0;
-                const uint64_t x = keys[lo], y = keys[hi];
-                if ((x < y) == desc) { keys[lo] = y; keys[hi] = x; }
+    if (need <= 64u) {
+        // Few keys wanted: every wave sorts a chunk of its own, no barrier inside (LDS serves a
+        // wave's requests in order), and a tree of merges -- the 64 larger of two sorted 64s form
+        // a bitonic run, six strides sort it -- leaves the 64 best of all in front.
+        const uint32_t lane = uint32_t(t) & 63u, wv = uint32_t(t) >> 6;
+        const uint32_t len = max(64u, sort_n / (kFinalThreads / 64));
+        const uint32_t n_chunks = sort_n / len;
+        auto wave_sync = []() {
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        };
+        auto swap_down = [&](uint32_t lo, uint32_t hi) {   // larger key to the lower index
+            const uint64_t x = keys[lo], y = keys[hi];
+            if (x < y) { keys[lo] = y; keys[hi] = x; }
+        };
+        if (wv < n_chunks) {
+            const uint32_t at = wv * len;
+            for (uint32_t size = 2; size <= len; size <<= 1) {
+                for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+                    for (uint32_t i = lane; i < len / 2; i += 64) {
+                        const uint32_t lo = 2 * i - (i & (stride - 1));
+                        const uint32_t hi = lo + stride;
+                        if ((lo & size) == 0) swap_down(at + lo, at + hi);
+                        else swap_down(at + hi, at + lo);
+                    }
+                    wave_sync();
+                }
             }
+        }
+        for (uint32_t step = 1; step < n_chunks; step <<= 1) {
             __syncthreads();
+            if (wv % (2 * step) == 0 && wv + step < n_chunks) {
+                const uint32_t at = wv * len, other = (wv + step) * len;
+                const uint64_t x = keys[at + lane], y = keys[other + 63u - lane];
+                if (x < y) keys[at + lane] = y;
+                wave_sync();
+                for (uint32_t stride = 32; stride > 0; stride >>= 1) {
+                    if (lane < 32u) {
+                        const uint32_t lo = 2 * lane - (lane & (stride - 1));
+                        swap_down(at + lo, at + lo + stride);
+                    }
+                    wave_sync();
+                }
+            }
+        }
+        __syncthreads();
+    } else {
+        for (uint32_t size = 2; size <= sort_n; size <<= 1) {
+            for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+                for (uint32_t i = t; i < sort_n / 2; i += kFinalThreads) {
+                    const uint32_t lo = 2 * i - (i & (stride - 1));
+                    const uint32_t hi = lo + stride;
+                    const bool desc = (lo & size) == 0;
+                    const uint64_t x = keys[lo], y = keys[hi];
+                    if ((x < y) == desc) { keys[lo] = y; keys[hi] = x; }
+                }
+                __syncthreads();
+            }
         }
     }
     if (sampling) {
