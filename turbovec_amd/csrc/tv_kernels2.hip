@@ -185,7 +185,7 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
     uint4 buf[U];
     if (j < j_end) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(j) * step * nch + u) * 64];
+        for (int u = 0; u < U; ++u) buf[u] = load_stream16(&codes[(size_t(j) * step * nch + u) * 64]);
     }
     while (j < j_end) {
         const uint32_t nj_live = live_from(j + total_waves);
@@ -205,10 +205,10 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
             for (int u = 0; u < U; ++u) cur[u] = buf[u];
             if (c0 + U < nch) {
 #pragma unroll
-                for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(b) * nch + c0 + U + u) * 64];
+                for (int u = 0; u < U; ++u) buf[u] = load_stream16(&codes[(size_t(b) * nch + c0 + U + u) * 64]);
             } else if (nj_live < j_end) {
 #pragma unroll
-                for (int u = 0; u < U; ++u) buf[u] = codes[(size_t(nj_live) * step * nch + u) * 64];
+                for (int u = 0; u < U; ++u) buf[u] = load_stream16(&codes[(size_t(nj_live) * step * nch + u) * 64]);
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {

@@ -33,7 +33,7 @@ __device__ __forceinline__ void dma16_to_lds(uint32_t lds_addr, const void *sbas
 // 16 bytes per lane from uniform base + 16 * lane into registers, invisible to the compiler's
 // wait-count bookkeeping (wait_vm<N> on the destination is the matching wait).
 __device__ __forceinline__ void load16_async_s(u32x4 &dst, const void *sbase, uint32_t lane16) {
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(dst) : "v"(lane16), "s"(sbase));
+    asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(dst) : "v"(lane16), "s"(sbase));
 }
 
 // 16 bytes of LDS per lane, requested without telling the compiler's wait-count bookkeeping;
