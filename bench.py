@@ -34,7 +34,7 @@ sys.path.insert(0, ROOT)
 # HBM bytes one launch of the dominant kernel moves (reads + writes), from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this same command, each scaled by the copy-probe factor (see profiles/).
 MEASURED_TRAFFIC = {
-    ("k_scan_p4_wide", 10_000_000, 1536, 4): 8.7075e9,    # 4,222,063 x 2 KiB fetched + 59,320 KiB written
+    ("k_scan_p4_wide", 10_000_000, 1536, 4): 7.7957e9,    # 3,775,883 x 2 KiB fetched + 61,218 KiB written
     ("k_scan_p4_multi", 10_000_000, 1536, 4): 7.7385e9,   # 3,775,909 x 2 KiB fetched + 5,261 KiB written
     ("k_scan_p4", 10_000_000, 1536, 4): 7.7206e9,         # 3,769,793 x 2 KiB fetched + 68 KiB written
 }
