@@ -2,25 +2,34 @@
 // every query of the chunk (up to 1024), not one group of tiles per pass.
 //
 // A wave decodes its 32-vector block once into registers -- the int8 A operands
-// of all its chunks, 8 VGPRs per chunk -- and keeps them there while the
+// of all its chunks, 8 registers per chunk -- and keeps them there while the
 // workgroup walks the query tiles: each tile's weights stream from L2 into LDS
-// in half-tile slices through a ring of LDS slots, requested four slices ahead
-// by direct-to-LDS loads that use no registers; a slice is NCH/2 chunks, i.e. NCH MFMAs per wave against B
-// operands read from LDS.  The nibble decode and the HBM read of the codes are
-// paid once per block instead of once per 96 queries, which leaves the matrix
-// unit as the bound: 2 * 32 * 32 * 32 * NCH * 2 int8 operations per (block, tile).
+// in slices (half a tile, or a quarter for long rows) through a ring of LDS
+// slots, requested four slices ahead by direct-to-LDS loads that use no
+// registers; the hand-over of a slice sits in the middle of the previous
+// slice's MFMAs.  B operands are read from LDS in one explicitly pipelined
+// stream.  The nibble decode and the HBM read of the codes are paid once per
+// block instead of once per 96 queries, which leaves the matrix unit as the
+// bound: 2 * 32 * 32 * 32 * NCH * 2 int8 operations per (block, tile).
+//
+// Three shapes of one template: rows of 16 to 24 chunks, one block per wave, 8
+// waves per workgroup at 256 registers; rows of 32 to 48 chunks, 4 waves at 512
+// registers (A operands partly in AGPRs); rows of 4 to 12 chunks, 2 to 4 blocks
+// per wave, every B operand feeding as many MFMAs.
 //
 // Integers and float epilogue are those of k_scan_p4 (turbovec/src/search.rs:
 // 1392-1567, 1519-1524); only the order in which (block, tile) pairs are visited
-// differs, and the candidate segments make the result independent of it.
+// differs, and the candidate segments make the result independent of it.  The
+// float epilogue is skipped for a tile whose accumulators all stay below an
+// integer bound that no passing score can stay below (WideQuery).
 #include "tv_device.h"
 #include "tv_internal.h"
 
 namespace tv {
 
-constexpr int kWideThreads = 512;    // 8 waves, 2 per SIMD: one wave's epilogue and decode run under the other's MFMAs
+constexpr int kWideThreads = 512;    // the widest form (and the matrix-unit probe): 8 waves, 2 per SIMD
 constexpr int kWideWaves = kWideThreads / 64;
-constexpr int kWideRing = 5;         // LDS slots of half a tile each; kWideRing - 1 slices are requested ahead
+constexpr int kWideRing = 5;         // LDS slots of one slice each; kWideRing - 1 slices are requested ahead
 
 // 16 bytes per lane from global memory (uniform base + 16 * lane) straight into LDS at
 // lds_addr + 16 * lane (lds_addr uniform over the wave).  Counted by the vector-memory counter
