@@ -920,7 +920,7 @@ __global__ __launch_bounds__(256) void k_merge(const float *__restrict__ part_sc
 // ===========================================================================
 
 constexpr int kFinalThreads = 1024;
-constexpr int kFinalLong = kFinalCap / 4;   // segments of more than 4 keys that fit the sort buffer
+constexpr int kFinalLong = kFinalCap / 8;   // segments of more than 8 keys that fit the sort buffer
 
 __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restrict__ cand,
                                                const uint32_t *__restrict__ cand_cnt, uint32_t n_seg,
@@ -931,7 +931,7 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
     __shared__ uint64_t keys[kFinalCap];
     __shared__ uint32_t wave_sum[kFinalThreads / 64];
     __shared__ uint32_t any_full, long_n;
-    __shared__ uint32_t long_seg[kFinalLong], long_pos[kFinalLong];
+    __shared__ uint32_t long_seg[kFinalLong], long_pos[kFinalLong], long_cnt[kFinalLong];
     const int qn = blockIdx.x;
     const int t = threadIdx.x;
     const bool sampling = tau_out != nullptr;
@@ -970,24 +970,26 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
     }
     // gather (a sampling level may keep any subset: dropping what does not fit only loosens the floor).
     // A thread copies a short segment itself, its loads in flight together; long ones (the first
-    // sampling level fills a few segments to the brim) go on a list the waves then share, a
-    // segment per wave and turn, a key per lane.
+    // sampling level fills a few segments to the brim) go on a list the waves then share, four
+    // segments per wave and turn, a key per lane.
     uint32_t pos = base;
+    constexpr uint32_t kShort = 8;
     for (uint32_t sg = s0; sg < s1; ++sg) {
         const uint32_t c = min(cnt[sg], uint32_t(kSegCap));
         const uint64_t *src = cand + (size_t(qn) * seg_stride + sg) * kSegCap;
-        if (c <= 4) {
-            uint64_t v[4];
+        if (c <= kShort) {
+            uint64_t v[kShort];
 #pragma unroll
-            for (uint32_t e = 0; e < 4; ++e) v[e] = e < c ? src[e] : 0ull;
+            for (uint32_t e = 0; e < kShort; ++e) v[e] = e < c ? src[e] : 0ull;
 #pragma unroll
-            for (uint32_t e = 0; e < 4; ++e)
+            for (uint32_t e = 0; e < kShort; ++e)
                 if (e < c && pos + e < uint32_t(kFinalCap)) keys[pos + e] = v[e];
         } else {
             const uint32_t slot = atomicAdd(&long_n, 1u);
             if (slot < uint32_t(kFinalLong)) {
                 long_seg[slot] = sg;
                 long_pos[slot] = pos;
+                long_cnt[slot] = c;
             } else {                      // more long segments than the list holds: copy in place
                 for (uint32_t e = 0; e < c; ++e)
                     if (pos + e < uint32_t(kFinalCap)) keys[pos + e] = src[e];
@@ -997,11 +999,26 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
     }
     __syncthreads();
     const uint32_t n_long = min(long_n, uint32_t(kFinalLong));
-    for (uint32_t i = uint32_t(t >> 6); i < n_long; i += kFinalThreads / 64) {
-        const uint32_t sg = long_seg[i], at = long_pos[i] + uint32_t(t & 63);
-        const uint32_t c = min(cnt[sg], uint32_t(kSegCap));
-        if (uint32_t(t & 63) < c && at < uint32_t(kFinalCap))
-            keys[at] = cand[(size_t(qn) * seg_stride + sg) * kSegCap + (t & 63)];
+    constexpr uint32_t kWavesF = kFinalThreads / 64;
+    for (uint32_t i0 = uint32_t(t >> 6); i0 < n_long; i0 += kWavesF * 4) {   // four segments' loads in flight per wave
+        uint64_t v[4];
+        uint32_t at[4];
+        bool ok[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const uint32_t i = i0 + u * kWavesF;
+            ok[u] = false;
+            at[u] = 0;
+            v[u] = 0ull;
+            if (i < n_long) {
+                at[u] = long_pos[i] + uint32_t(t & 63);
+                ok[u] = uint32_t(t & 63) < long_cnt[i] && at[u] < uint32_t(kFinalCap);
+                if (ok[u]) v[u] = cand[(size_t(qn) * seg_stride + long_seg[i]) * kSegCap + (t & 63)];
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+            if (ok[u]) keys[at[u]] = v[u];
     }
     const uint32_t c_all = min(total, uint32_t(kFinalCap));
     const uint32_t need = sampling ? min(uint32_t(k_floor), c_all) : uint32_t(k_eff);   // leading keys wanted, in order
