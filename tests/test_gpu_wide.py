@@ -117,3 +117,47 @@ def test_wide_scan_with_wild_row_scales(T, oracle):
         assert np.array_equal(i, i2) and bits_equal(s, s2), k
         assert np.array_equal(i, i3) and bits_equal(s, s3), k
     ix.close()
+
+
+# batch_matches_single.rs / kernel_correctness.rs:268-312, for batches that take the wide kernel:
+# every row of the batch equals the same query searched alone (another kernel), ids and score bits;
+# query_scale_invariance.rs: ids survive a power-of-two scaling of the queries
+def test_wide_batch_equals_single_and_scale_invariance(T, oracle):
+    dim, n = 1536, 4_003
+    oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=51))
+    ix = to_native(T, oidx)
+    q = unit_gaussian(130, dim, seed=52)
+    s, i = ix.search(q, 10)
+    assert ix.queries_per_launch() == 130
+    for qi in range(0, 130, 7):
+        s1, i1 = ix.search(q[qi:qi + 1], 10)
+        assert np.array_equal(i1[0], i[qi]) and bits_equal(s1[0], s[qi])
+    for e in (-60, -20, 10, 40):
+        _, i2 = ix.search(q * np.float32(2.0 ** e), 10)
+        assert np.array_equal(i2, i)
+    ix.close()
+
+
+# concurrent_search.rs: threads searching one index at once see identical results
+def test_wide_concurrent_searches(T, oracle):
+    import threading
+    dim, n = 1280, 3_001
+    oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=53))
+    ix = to_native(T, oidx)
+    q = unit_gaussian(150, dim, seed=54)
+    want_s, want_i = ix.search(q, 10)
+    bad = []
+
+    def worker():
+        for _ in range(6):
+            s, i = ix.search(q, 10)
+            if not (np.array_equal(i, want_i) and bits_equal(s, want_s)):
+                bad.append(1)
+
+    threads = [threading.Thread(target=worker) for _ in range(6)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not bad
+    ix.close()
