@@ -30,7 +30,9 @@ def masks_for(T, n, seed):
 @pytest.mark.parametrize("dim,n,nq", [(1536, 6_007, 300), (1280, 4_001, 257), (1280, 3_001, 100), (1024, 5_003, 520), (1536, 3_001, 1029),
                                       (2048, 3_001, 200), (2560, 2_001, 100), (3072, 2_501, 260),
                                       (256, 20_011, 333), (384, 9_001, 130), (512, 12_345, 200), (768, 7_003, 290),
-                                      (1024, 4_001, 129)])
+                                      (1024, 4_001, 129), (128, 30_011, 400), (640, 5_003, 140), (896, 4_001, 200),
+                                      (1152, 3_001, 130), (1408, 3_003, 100), (1792, 2_001, 100), (2304, 2_003, 129),
+                                      (2816, 1_501, 160)])
 def test_wide_scan_matches_oracle(T, oracle, dim, n, nq):
     oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=dim + n))
     q = unit_gaussian(nq, dim, seed=77)

@@ -383,9 +383,9 @@ hipError_t launch_probe_mfma(int device, int iters, uint32_t *sink, double *ops,
 // too, it is level at 128 queries and 1.6 to 1.7 times faster at 1024.
 int wide_min_queries(int nch) {
     switch (nch) {
-        case 4: case 6: case 8: case 12: case 16: return 129;
-        case 20: case 24: return 97;
-        case 32: case 40: case 48: return 97;
+        case 2: case 4: case 6: case 8: case 10: case 12: case 14: case 16: case 18: return 129;
+        case 20: case 22: case 24: return 97;
+        case 28: case 32: case 36: case 40: case 44: case 48: return 97;
         default: return 0;
     }
 }
@@ -419,16 +419,25 @@ static hipError_t launch_wide_n(const ScanArgs &a, int grid, hipStream_t s) {
 // ceil(nq/32) weight tiles back to back, a.qscale / a.qbias / a.gtau indexed by query.
 hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s) {
     switch (a.nch) {
+        // <chunks, B-operand registers, waves, slices per tile, blocks per wave>
+        case 2: return launch_wide_n<2, 2, 8, 1, 6>(a, grid, s);
         case 4: return launch_wide_n<4, 2, 8, 1, 4>(a, grid, s);
         case 6: return launch_wide_n<6, 2, 8, 1, 3>(a, grid, s);
         case 8: return launch_wide_n<8, 4, 8, 1, 2>(a, grid, s);
+        case 10: return launch_wide_n<10, 2, 8, 2, 2>(a, grid, s);
         case 12: return launch_wide_n<12, 2, 8, 2, 2>(a, grid, s);
-        case 16: return launch_wide_n<16, 4>(a, grid, s);
-        case 20: return launch_wide_n<20, 4>(a, grid, s);
-        case 24: return launch_wide_n<24, 2>(a, grid, s);
-        case 32: return launch_wide_n<32, 4, 4, 4>(a, grid, s);
-        case 40: return launch_wide_n<40, 4, 4, 4>(a, grid, s);
-        case 48: return launch_wide_n<48, 4, 4, 4>(a, grid, s);
+        case 14: return launch_wide_n<14, 2, 8, 2, 1>(a, grid, s);
+        case 16: return launch_wide_n<16, 4, 8, 2, 1>(a, grid, s);
+        case 18: return launch_wide_n<18, 2, 8, 2, 1>(a, grid, s);
+        case 20: return launch_wide_n<20, 4, 8, 2, 1>(a, grid, s);
+        case 22: return launch_wide_n<22, 2, 8, 2, 1>(a, grid, s);
+        case 24: return launch_wide_n<24, 2, 8, 2, 1>(a, grid, s);
+        case 28: return launch_wide_n<28, 2, 4, 4, 1>(a, grid, s);
+        case 32: return launch_wide_n<32, 4, 4, 4, 1>(a, grid, s);
+        case 36: return launch_wide_n<36, 2, 4, 4, 1>(a, grid, s);
+        case 40: return launch_wide_n<40, 4, 4, 4, 1>(a, grid, s);
+        case 44: return launch_wide_n<44, 2, 4, 4, 1>(a, grid, s);
+        case 48: return launch_wide_n<48, 4, 4, 4, 1>(a, grid, s);
         default: return hipErrorInvalidValue;
     }
 }
