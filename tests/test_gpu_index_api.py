@@ -278,3 +278,32 @@ def test_calibrate_before_add(api):
         api.TurboQuantIndex(256, 4).calibrate(v[:1])
     with pytest.raises(TypeError):
         api.TurboQuantIndex(256, 4).calibrate(v.astype(np.float64))
+
+
+# test_pickle_copy.py in the reference's Python suite: pickle / copy / deepcopy go through
+# from_bytes(to_bytes()) and yield an independent index with the same answers
+def test_pickle_and_copy_round_trip(api):
+    import copy
+    import pickle
+    TurboQuantIndex, IdMapIndex = api.TurboQuantIndex, api.IdMapIndex
+    rng = np.random.default_rng(21)
+    v = rng.standard_normal((300, 64)).astype(np.float32)
+    q = rng.standard_normal((3, 64)).astype(np.float32)
+    idx = TurboQuantIndex(dim=64, bit_width=4)
+    idx.add(v)
+    want = idx.search(q, 5)
+    for clone in (pickle.loads(pickle.dumps(idx)), copy.copy(idx), copy.deepcopy(idx)):
+        assert len(clone) == 300 and clone.to_bytes() == idx.to_bytes()
+        got = clone.search(q, 5)
+        assert np.array_equal(got[1], want[1]) and np.array_equal(got[0], want[0])
+    clone = copy.deepcopy(idx)
+    clone.swap_remove(0)
+    assert len(idx) == 300 and len(clone) == 299          # independent of the original
+    im = IdMapIndex(dim=64, bit_width=2)
+    ids = np.arange(1000, 1300, dtype=np.uint64)
+    im.add_with_ids(v, ids)
+    want = im.search(q, 5)
+    clone = pickle.loads(pickle.dumps(im))
+    got = clone.search(q, 5)
+    assert np.array_equal(got[1], want[1]) and np.array_equal(got[0], want[0])
+    assert clone.contains(1005) and not clone.contains(5)

@@ -126,6 +126,12 @@ class TurboQuantIndex:
     def from_bytes(cls, data, device=0):
         return cls._adopt(*_load_image(data, device, want_kind=0))
 
+    def __reduce__(self):
+        """pickle, copy.copy and copy.deepcopy rebuild through from_bytes(to_bytes()), as the
+        reference's bindings do (turbovec-python/src/lib.rs:268-287, 828-833): the copy is a
+        separate index with its own device memory."""
+        return (type(self).from_bytes, (self.to_bytes(),))
+
     @classmethod
     def _adopt(cls, native, _ids):
         self = cls.__new__(cls)
@@ -260,6 +266,10 @@ class IdMapIndex:
         if len(self._id_to_slot) != len(self._slot_to_id):
             raise OSError("image holds duplicate ids")
         return self
+
+    def __reduce__(self):
+        """See TurboQuantIndex.__reduce__ (turbovec-python/src/lib.rs:1462-1468)."""
+        return (type(self).from_bytes, (self.to_bytes(),))
 
     def write(self, path):
         _write_atomically(path, self.to_bytes())
