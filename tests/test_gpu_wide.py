@@ -163,3 +163,49 @@ def test_wide_concurrent_searches(T, oracle):
         t.join()
     assert not bad
     ix.close()
+
+
+# seeded sweep over row lengths (with and without a wide-kernel instance), sizes the oracle
+# cannot reach in seconds, batch sizes around the switch-over points, k around the selection
+# paths' limits, norm spread, duplicate rows (ties) and masks: the three search paths -- all
+# queries per pass, tile groups, exact lists / radix select -- must agree bit for bit
+def test_paths_agree_on_random_shapes(T):
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(2024)
+    dims = [128, 256, 384, 512, 640, 768, 896, 1024, 1152, 1280, 1408, 1536, 1792, 2048, 2304, 2560, 2816, 3072,
+            320, 1600]
+    for case in range(24):
+        dim = int(rng.choice(dims))
+        n = int(rng.integers(50, 120_000 if dim <= 1536 else 50_000))
+        nq = int(rng.choice([97, 128, 129, 130, 200, 257, 333, 512, 777, 1024, 1025]))
+        k = int(rng.choice([1, 10, 16, 64, 65, 100, 300]))
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(case * 7919 + 1)
+        ix = T.NativeIndex(dim, 4)
+        v = torch.randn(n, dim, device=dev, generator=gen)
+        if rng.random() < 0.3:
+            v *= torch.exp(torch.randn(n, 1, device=dev, generator=gen))
+        if rng.random() < 0.2:
+            v[: n // 3] = v[n // 3: 2 * (n // 3)]
+        torch.cuda.synchronize()
+        ix.add_dev(v.data_ptr(), n)
+        q = torch.randn(nq, dim, device=dev, generator=gen).cpu().numpy()
+        kind = int(rng.integers(0, 4))
+        m = None
+        if kind == 1:
+            m = rng.random(n) < rng.choice([0.5, 0.05, 0.002])
+        elif kind == 2:
+            lo = int(rng.integers(0, n))
+            m = (np.arange(n) >= lo) & (np.arange(n) < lo + max(1, n // 20))
+        elif kind == 3:
+            m = np.zeros(n, bool)
+            m[rng.integers(0, n, size=min(n, 7))] = True
+        words = None if m is None else T.pack_mask(m)[0]
+        res = []
+        for path in (0, 4, 1):
+            ix.set_path(path)
+            res.append(ix.search(q, k, mask_words=words))
+        for s, i in res[1:]:
+            assert np.array_equal(res[0][1], i) and bits_equal(res[0][0], s), (case, dim, n, nq, k, kind)
+        ix.close()
+        del v
