@@ -16,28 +16,43 @@
  *                            the encode fingerprint codes/scales hashes.
  *   tvo_codebook             pinned: FNV-1a-64 of boundaries/centroids for 8
  *                            (dim,bits) cells (tests/encode_fingerprint.rs:83-92).
- *                            (128,4) has no golden: PARITY UNPINNED for that cell
- *                            beyond ordering/symmetry/midpoint invariants.
+ *                            Cells without a golden, (128,4) among them: an
+ *                            independent Lloyd-Max (cell probabilities from scipy's
+ *                            incomplete beta function, conditional means in closed
+ *                            form, no quadrature) reproduces the golden hashes and
+ *                            equals this function bit for bit in every cell.
  *   tvo_fit_calibration,
  *   tvo_encode, tvo_norm     pinned: calibration/codes/scales hashes, 8 cells.
  *   tvo_repack_seq et al.    pinned: closed-form byte maps (src/pack.rs:964-1008).
- *   tvo_build_lut            pinned end to end through the parity fixture below (any
- *                            wrong entry, scale or bias moves one of its 600 floats);
- *                            2-/3-bit tables: PARITY UNPINNED beyond invariants
- *                            (entries <= 127, power-of-two scaling, zero query).
+ *   tvo_build_lut            pinned end to end at 4-bit through the parity fixture below
+ *                            (any wrong entry, scale or bias moves one of its 600
+ *                            floats); at 2, 3 and 4 bits every byte, the scale and the
+ *                            bias equal an independent numpy float32 model.
  *   tvo_search  L_CLASSIC    pinned at 4-bit: the 3 x 200 float scores and ids of
  *                            benchmarks/hillclimb/data/parity_base_{x86,arm}.json are
  *                            reproduced bit for bit (base, after the warm appends,
  *                            after 500 swap-removes).
- *   tvo_build_permute_dot    slot map and zero identity pinned (src/search.rs:4596);
- *   tvo_search  mode P       end-to-end floats PARITY UNPINNED: the reference holds no
- *                            vector produced by its int8 permute-dot kernel (the fixture
- *                            above was written by the LUT kernel).  Integer dots are
- *                            checked by brute force against decoded codes; ranking
- *                            agrees with the fixture up to quantisation of the weights.
- *   tvo_search  L_U32,       PARITY UNPINNED end to end; they share the pinned LUT and
- *               L_SCALAR     integer sums with L_CLASSIC, the epilogue follows
- *                            search.rs:1174-1177 / 3077-3147 line by line.
+ *   tvo_build_permute_dot    pinned: slot map and zero identity (src/search.rs:4596);
+ *                            every weight, level, zero and scale equal an independent
+ *                            numpy float32 model over 360 queries (dims 128/1536/3072),
+ *                            half-way values (round half away from zero) and the
+ *                            +-127 ends included.
+ *   tvo_calibrate_query      pinned: exact-rational model of the sequential f64 sum
+ *                            (inputs chosen so that a float32 accumulator, an exactly
+ *                            rounded sum, the reversed order and the opposite sign all
+ *                            give another answer).
+ *   tvo_search  mode P,      pinned: the reference holds no vector written by these
+ *               L_U32,       kernels (the fixture above was written by the classic LUT
+ *               L_SCALAR     kernel), so every float score is compared with an
+ *                            exact-rational evaluation of its epilogue, each IEEE
+ *                            operation rounded once (P: fma(f32(acc), scale, bias) *
+ *                            row scale, |acc| > 2^24 included; L_U32: multiply, add,
+ *                            multiply; L_SCALAR: two multiply-adds per group), on
+ *                            TQ+-calibrated indexes so the bias is not zero and fused
+ *                            and unfused forms differ; integers by brute force over
+ *                            decoded codes; scores estimate true inner products to
+ *                            quantisation noise (src/kernel_tests.rs:401-419).
+ *                            All of this lives in tests/test_oracle_pins.py.
  */
 #ifndef TV_ORACLE_H
 #define TV_ORACLE_H
