@@ -144,6 +144,8 @@ def main():
 
     def run(nq, steps, warmup):
         q = make_queries(nq)
+        # the library works on its own stream: buffers handed to a _dev entry point must be complete
+        torch.cuda.synchronize()
         out_s = torch.empty(nq, k, device=dev)
         out_i = torch.empty(nq, k, dtype=torch.int64, device=dev)
         for _ in range(warmup):

@@ -15,6 +15,13 @@
  * the reference's `&mut self` methods do; tv_search* may be called from many
  * threads at once (calls on one index are serialised internally).  A process
  * that has used the library must not fork() and keep using it in the child.
+ *
+ * Device buffers (_dev entry points, device pointers): the library runs on a
+ * stream of its own per index, not on the caller's.  Every device buffer handed
+ * in must be complete -- the work that writes it finished, e.g. the producing
+ * stream synchronised -- before the call, and must stay untouched until the call
+ * returns; outputs are complete when the call returns (it synchronises its
+ * stream before returning).
  */
 #ifndef TURBOVEC_HIP_H
 #define TURBOVEC_HIP_H

@@ -71,7 +71,13 @@ int ensure_capacity(tv_index *ix, size_t n_vectors) {
     float *scales = nullptr;
     const size_t bb = ix->geo.block_bytes();
     TV_HIP(hipMalloc(reinterpret_cast<void **>(&codes), cap * bb));
-    TV_HIP(hipMalloc(reinterpret_cast<void **>(&scales), cap * tv::kVecBlock * sizeof(float)));
+    {
+        const hipError_t e = hipMalloc(reinterpret_cast<void **>(&scales), cap * tv::kVecBlock * sizeof(float));
+        if (e != hipSuccess) {
+            (void)hipFree(codes);
+            return fail_hip(e, "hipMalloc(scales)");
+        }
+    }
     const size_t old_blocks = (ix->n + tv::kVecBlock - 1) / tv::kVecBlock;
     // fresh bytes are zero so padding lanes match a from-scratch upload
     TV_HIP(hipMemsetAsync(codes + old_blocks * bb, 0, (cap - old_blocks) * bb, ix->stream));
@@ -88,6 +94,18 @@ int ensure_capacity(tv_index *ix, size_t n_vectors) {
     ix->d_codes = codes;
     ix->d_scales = scales;
     ix->cap_blocks = cap;
+    return TV_OK;
+}
+
+// An upload replaces the contents: blocks of the old contents beyond the new end are cleared, so
+// that rows appended later land in zeroed blocks (padding lanes zero, as in a from-scratch
+// upload; pack.rs:235-243, :354).
+int clear_tail_blocks(tv_index *ix, size_t n_blocks) {
+    if (n_blocks >= ix->cap_blocks) return TV_OK;
+    const size_t bb = ix->geo.block_bytes();
+    TV_HIP(hipMemsetAsync(ix->d_codes + n_blocks * bb, 0, (ix->cap_blocks - n_blocks) * bb, ix->stream));
+    TV_HIP(hipMemsetAsync(ix->d_scales + n_blocks * tv::kVecBlock, 0,
+                          (ix->cap_blocks - n_blocks) * tv::kVecBlock * sizeof(float), ix->stream));
     return TV_OK;
 }
 
@@ -190,20 +208,17 @@ constexpr size_t kChunkQueries = 1024;
 constexpr size_t kTauOpenInts = kChunkQueries * tv::kQTile;
 constexpr int kMaxTimedTiles = int(kChunkQueries / tv::kQTile);
 
-struct EventPool {
-    hipEvent_t start[kMaxTimedTiles];
-    hipEvent_t stop[kMaxTimedTiles];
-    bool ready = false;
-};
-thread_local EventPool g_events;
+static_assert(kMaxTimedTiles == tv::kTimedLaunches, "the index holds one event pair per timed launch");
 
-int ensure_events() {
-    if (g_events.ready) return TV_OK;
+// The events that time scan launches belong to the index (created on first use under its lock,
+// destroyed with it).
+int ensure_events(tv_index *ix) {
+    if (ix->events_ready) return TV_OK;
     for (int i = 0; i < kMaxTimedTiles; ++i) {
-        TV_HIP(hipEventCreate(&g_events.start[i]));
-        TV_HIP(hipEventCreate(&g_events.stop[i]));
+        TV_HIP(hipEventCreate(&ix->ev_start[i]));
+        TV_HIP(hipEventCreate(&ix->ev_stop[i]));
     }
-    g_events.ready = true;
+    ix->events_ready = true;
     return TV_OK;
 }
 
@@ -268,10 +283,10 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
                 TV_HIP(tv::launch_fill_i32(reinterpret_cast<int *>(d_dense), 0x7fc00000, size_t(a.nq_tile) * n, ix->stream));
             const bool timed = timed_run && int(t) < kMaxTimedTiles;
             const int smode = lists ? tv::kModeLists : tv::kModeDump;
-            if (timed) TV_HIP(hipEventRecord(g_events.start[t], ix->stream));
+            if (timed) TV_HIP(hipEventRecord(ix->ev_start[t], ix->stream));
             if (mode_p) TV_HIP(tv::launch_scan_p4(a, grid, smode, ix->stream));
             else TV_HIP(tv::launch_scan_lut(a, grid, smode, ix->stream));
-            if (timed) TV_HIP(hipEventRecord(g_events.stop[t], ix->stream));
+            if (timed) TV_HIP(hipEventRecord(ix->ev_stop[t], ix->stream));
             float *os = d_out_scores + (q0 + t * tile_q) * k_eff;
             int64_t *oi = d_out_idx + (q0 + t * tile_q) * k_eff;
             if (lists) {
@@ -285,7 +300,7 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
         TV_HIP(hipStreamSynchronize(ix->stream));
         for (size_t t = 0; timed_run && t < n_tiles && int(t) < kMaxTimedTiles; ++t) {
             float ms = 0.0f;
-            TV_HIP(hipEventElapsedTime(&ms, g_events.start[t], g_events.stop[t]));
+            TV_HIP(hipEventElapsedTime(&ms, ix->ev_start[t], ix->ev_stop[t]));
             ix->last_scan_ms += ms;
             ix->last_scan_launches += 1;
         }
@@ -342,7 +357,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
     const int mode = effective_mode(ix);
     if (mode == TV_SCORE_P && g.bits != 4) { g_last_error = "score mode P needs 4-bit codes"; return TV_ERR_BAD_ARGUMENT; }
     const bool mode_p = mode == TV_SCORE_P;
-    int rc = ensure_events();
+    int rc = ensure_events(ix);
     if (rc != TV_OK) return rc;
     if (k_eff > size_t(tv::kMaxSampledK) || ix->force_robust)
         return search_robust(ix, d_queries, nq, k_eff, d_mask, d_out_scores, d_out_idx, true);
@@ -410,7 +425,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
                 a.cand_cnt = d_cnt + t * tile_q * seg_stride;
                 a.seg_stride = uint32_t(seg_stride);
                 const bool timed = last && int(launch_no) < kMaxTimedTiles;
-                if (timed) TV_HIP(hipEventRecord(g_events.start[launch_no], ix->stream));
+                if (timed) TV_HIP(hipEventRecord(ix->ev_start[launch_no], ix->stream));
                 if (wide) {
                     n_seg = grid;
                     TV_HIP(tv::launch_scan_p4_wide(a, n_seg, ix->stream));
@@ -422,19 +437,19 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
                 } else {
                     TV_HIP(tv::launch_scan_lut(a, lgrid, tv::kModeAppend, ix->stream));
                 }
-                if (timed) TV_HIP(hipEventRecord(g_events.stop[launch_no], ix->stream));
+                if (timed) TV_HIP(hipEventRecord(ix->ev_stop[launch_no], ix->stream));
             }
             if (last) n_timed = std::min<size_t>(launch_no, size_t(kMaxTimedTiles));
             TV_HIP(tv::launch_final(d_cand, d_cnt, uint32_t(n_seg), uint32_t(seg_stride), int(k_eff), int(k_floor),
                                     int(cq), d_out_scores + q0 * k_eff, d_out_idx + q0 * k_eff, d_over,
-                                    last ? nullptr : d_tau, int(tile_q), ix->stream));
+                                    last ? nullptr : d_tau, int(tile_q), lv > 0 ? 1 : 0, ix->stream));
         }
         h_over.resize(cq);
         TV_HIP(hipMemcpyAsync(h_over.data(), d_over, cq * sizeof(uint32_t), hipMemcpyDeviceToHost, ix->stream));
         TV_HIP(hipStreamSynchronize(ix->stream));
         for (size_t t = 0; t < n_timed; ++t) {
             float ms = 0.0f;
-            TV_HIP(hipEventElapsedTime(&ms, g_events.start[t], g_events.stop[t]));
+            TV_HIP(hipEventElapsedTime(&ms, ix->ev_start[t], ix->ev_stop[t]));
             ix->last_scan_ms += ms;
             ix->last_scan_launches += 1;
         }
@@ -534,6 +549,11 @@ int tv_index_destroy(tv_index *ix) {
     void *ptrs[] = {ix->d_signs, ix->d_perms, ix->d_centroids, ix->d_tq_shift, ix->d_tq_scale,
                     ix->d_codes, ix->d_scales, ix->ws, ix->io, ix->d_tau_open};
     for (void *p : ptrs) if (p) (void)hipFree(p);
+    if (ix->events_ready)
+        for (int i = 0; i < tv::kTimedLaunches; ++i) {
+            (void)hipEventDestroy(ix->ev_start[i]);
+            (void)hipEventDestroy(ix->ev_stop[i]);
+        }
     if (ix->stream) (void)hipStreamDestroy(ix->stream);
     delete ix;
     return TV_OK;
@@ -541,6 +561,7 @@ int tv_index_destroy(tv_index *ix) {
 
 int tv_index_set_tables(tv_index *ix, const float *signs, const uint32_t *perms, const float *centroids) {
     if (!ix) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
     TV_HIP(hipSetDevice(ix->device));
     const size_t dim = size_t(ix->geo.dim);
     if (signs) ix->rot.signs.assign(signs, signs + 2 * dim);
@@ -559,6 +580,7 @@ int tv_index_set_tables(tv_index *ix, const float *signs, const uint32_t *perms,
 
 int tv_index_set_calibration(tv_index *ix, const float *shift, const float *scale) {
     if (!ix || (shift == nullptr) != (scale == nullptr)) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
     TV_HIP(hipSetDevice(ix->device));
     const size_t dim = size_t(ix->geo.dim);
     if (!shift) { ix->tq_shift.clear(); ix->tq_scale.clear(); return TV_OK; }
@@ -575,6 +597,7 @@ int tv_index_set_score_mode(tv_index *ix, int mode) {
     if (mode != TV_SCORE_AUTO && mode != TV_SCORE_L_CLASSIC && mode != TV_SCORE_L_U32 && mode != TV_SCORE_P)
         return TV_ERR_BAD_ARGUMENT;
     if (mode == TV_SCORE_P && ix->geo.bits != 4) { g_last_error = "score mode P needs 4-bit codes"; return TV_ERR_BAD_ARGUMENT; }
+    std::lock_guard<std::mutex> lock(ix->mu);
     ix->score_mode = mode;
     return TV_OK;
 }
@@ -599,6 +622,8 @@ int tv_index_upload_seq(tv_index *ix, const uint8_t *seq_codes, size_t n_vectors
     const tv::Geometry &g = ix->geo;
     const size_t n_blocks = (n_vectors + tv::kVecBlock - 1) / tv::kVecBlock;
     const size_t seq_block = size_t(g.G) * tv::kVecBlock;
+    rc = clear_tail_blocks(ix, n_blocks);
+    if (rc != TV_OK) return rc;
     // stage the sequential-blocked bytes through the workspace in slices
     const size_t slice_blocks = std::max<size_t>(1, (size_t(256) << 20) / seq_block);
     rc = ensure_workspace(ix, std::min(n_blocks, slice_blocks) * seq_block + 256);
@@ -628,6 +653,8 @@ int tv_index_upload_seq_dev(tv_index *ix, const uint8_t *d_seq_codes, size_t n_v
     if (rc != TV_OK) return rc;
     const size_t n_blocks = (n_vectors + tv::kVecBlock - 1) / tv::kVecBlock;
     const size_t seq_block = size_t(ix->geo.G) * tv::kVecBlock;
+    rc = clear_tail_blocks(ix, n_blocks);
+    if (rc != TV_OK) return rc;
     const size_t slice_blocks = std::max<size_t>(1, (size_t(1) << 30) / seq_block);  // keeps each grid small
     for (size_t b0 = 0; b0 < n_blocks; b0 += slice_blocks) {
         const size_t nb = std::min(slice_blocks, n_blocks - b0);
@@ -1083,18 +1110,18 @@ int tv_debug_stream_probe(tv_index *ix, const void *d_src, void *d_dst, size_t b
     if (!ix || !d_src || reps <= 0) return TV_ERR_BAD_ARGUMENT;
     std::lock_guard<std::mutex> lock(ix->mu);
     TV_HIP(hipSetDevice(ix->device));
-    int rc = ensure_events();
+    int rc = ensure_events(ix);
     if (rc != TV_OK) return rc;
     rc = ensure_workspace(ix, 4096);
     if (rc != TV_OK) return rc;
     uint32_t *sink = static_cast<uint32_t *>(ix->ws);
     TV_HIP(tv::launch_probe(d_src, d_dst, bytes, d_dst != nullptr, sink, ix->stream));  // warm
-    TV_HIP(hipEventRecord(g_events.start[0], ix->stream));
+    TV_HIP(hipEventRecord(ix->ev_start[0], ix->stream));
     for (int r = 0; r < reps; ++r) TV_HIP(tv::launch_probe(d_src, d_dst, bytes, d_dst != nullptr, sink, ix->stream));
-    TV_HIP(hipEventRecord(g_events.stop[0], ix->stream));
+    TV_HIP(hipEventRecord(ix->ev_stop[0], ix->stream));
     TV_HIP(hipStreamSynchronize(ix->stream));
     float ms = 0.0f;
-    TV_HIP(hipEventElapsedTime(&ms, g_events.start[0], g_events.stop[0]));
+    TV_HIP(hipEventElapsedTime(&ms, ix->ev_start[0], ix->ev_stop[0]));
     if (ms_per_rep) *ms_per_rep = ms / float(reps);
     return TV_OK;
 }
@@ -1103,19 +1130,19 @@ int tv_debug_mfma_probe(tv_index *ix, int iters, int reps, float *ms_per_rep, do
     if (!ix || iters <= 0 || reps <= 0) return TV_ERR_BAD_ARGUMENT;
     std::lock_guard<std::mutex> lock(ix->mu);
     TV_HIP(hipSetDevice(ix->device));
-    int rc = ensure_events();
+    int rc = ensure_events(ix);
     if (rc != TV_OK) return rc;
     rc = ensure_workspace(ix, 4096);
     if (rc != TV_OK) return rc;
     uint32_t *sink = static_cast<uint32_t *>(ix->ws);
     double ops = 0.0;
     TV_HIP(tv::launch_probe_mfma(ix->device, iters, sink, &ops, ix->stream));  // warm
-    TV_HIP(hipEventRecord(g_events.start[0], ix->stream));
+    TV_HIP(hipEventRecord(ix->ev_start[0], ix->stream));
     for (int r = 0; r < reps; ++r) TV_HIP(tv::launch_probe_mfma(ix->device, iters, sink, &ops, ix->stream));
-    TV_HIP(hipEventRecord(g_events.stop[0], ix->stream));
+    TV_HIP(hipEventRecord(ix->ev_stop[0], ix->stream));
     TV_HIP(hipStreamSynchronize(ix->stream));
     float ms = 0.0f;
-    TV_HIP(hipEventElapsedTime(&ms, g_events.start[0], g_events.stop[0]));
+    TV_HIP(hipEventElapsedTime(&ms, ix->ev_start[0], ix->ev_stop[0]));
     if (ms_per_rep) *ms_per_rep = ms / float(reps);
     if (ops_per_rep) *ops_per_rep = ops;
     return TV_OK;

@@ -106,21 +106,31 @@ __global__ __launch_bounds__(256) void k_encode(EncodeArgs a) {
     }
     __syncthreads();
 
-    // encode.rs:1442-1475: inner = <rotated, reconstruction> in f64, four chains by j % 4
-    double *terms = reinterpret_cast<double *>(enc_lds + 2 * dim);
-    for (int j = t; j < dim; j += 256) {
-        const float sh = a.shift ? a.shift[j] : 0.0f;
-        const float sc = a.scale ? a.scale[j] : 1.0f;
-        const float inv_sc = 1.0f / sc;                       // encode.rs:594
-        const double recon = double(s_cen[codes[j]]) * double(inv_sc) - double(sh);
-        terms[j] = double(B[j]) * recon;
+    // encode.rs:1442-1475: inner = <rotated, reconstruction> in f64, four chains by j % 4.
+    // The f64 products are parked piece by piece in what is left of A behind the codes
+    // (3 * dim bytes), so the kernel needs 8 * dim bytes of LDS whatever the row length; a
+    // chain walks its elements in rising order across the pieces, as in one sweep.
+    // (rows of 8 dimensions leave no room for one product per chain there: they use the four
+    // spare doubles behind B)
+    const int piece = dim >= 16 ? (3 * dim / 8) & ~3 : 4;
+    double *terms = dim >= 16 ? reinterpret_cast<double *>(reinterpret_cast<uint8_t *>(A) + dim)
+                              : reinterpret_cast<double *>(enc_lds + 2 * dim);
+    double ch = 0.0;
+    for (int j0 = 0; j0 < dim; j0 += piece) {
+        const int j1 = min(dim, j0 + piece);
+        for (int j = j0 + t; j < j1; j += 256) {
+            const float sh = a.shift ? a.shift[j] : 0.0f;
+            const float sc = a.scale ? a.scale[j] : 1.0f;
+            const float inv_sc = 1.0f / sc;                       // encode.rs:594
+            const double recon = double(s_cen[codes[j]]) * double(inv_sc) - double(sh);
+            terms[j - j0] = double(B[j]) * recon;
+        }
+        __syncthreads();
+        if (t < 4)
+            for (int j = j0 + t; j < j1; j += 4) ch = ch + terms[j - j0];
+        __syncthreads();
     }
-    __syncthreads();
-    if (t < 4) {
-        double ch = 0.0;
-        for (int j = t; j < dim; j += 4) ch = ch + terms[j];
-        dred[t] = ch;
-    }
+    if (t < 4) dred[t] = ch;
     __syncthreads();
     if (t == 0) {
         const double inner = (dred[0] + dred[1]) + (dred[2] + dred[3]);
@@ -138,6 +148,10 @@ __global__ __launch_bounds__(256) void k_encode(EncodeArgs a) {
     }
 }
 
+// A and B, one float row each; codes and the f64 products overlay A.  128 KiB at the largest
+// row the index accepts (16384 dimensions), inside the 160 KiB a workgroup may have.
+size_t encode_lds_bytes(int dim) { return size_t(2) * size_t(dim) * sizeof(float) + 4 * sizeof(double); }
+
 hipError_t launch_encode(const float *d_vecs, size_t n_new, size_t old_n, const float *d_signs,
                          const uint32_t *d_perms, const float *d_shift, const float *d_scale,
                          const float *centroids, const float *boundaries, const Geometry &g, int block,
@@ -152,7 +166,7 @@ hipError_t launch_encode(const float *d_vecs, size_t n_new, size_t old_n, const 
     a.inv_sqrt_block = inv_sqrt_block;
     a.nat = d_native; a.scales = d_scales; a.old_n = old_n; a.n_new = n_new;
     a.rot_out = d_rot_out;
-    const size_t lds = size_t(2) * g.dim * sizeof(float) + size_t(g.dim) * sizeof(double);   // A, B, f64 terms
+    const size_t lds = encode_lds_bytes(g.dim);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_encode),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));

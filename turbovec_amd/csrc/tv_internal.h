@@ -19,6 +19,7 @@ constexpr int kMaxListK = 32;    // largest k served by the per-lane lists
 constexpr int kSegCap = 64;      // candidate keys one workgroup may append per query and launch
 constexpr int kFinalCap = 8192;  // candidate keys per query the final sort holds (64 KiB of LDS)
 constexpr int kMaxSampledK = 512;   // largest k served by sample-then-filter
+constexpr int kTimedLaunches = 32;  // scan launches of one search that are timed with events
 
 // What a scan launch does with the scores it computes.
 enum { kModeLists = 0,   // per-lane top-k lists (written out for k_merge)
@@ -78,6 +79,7 @@ hipError_t launch_encode(const float *d_vecs, size_t n_new, size_t old_n, const 
                          const float *centroids, const float *boundaries, const Geometry &g, int block,
                          float inv_sqrt_block, uint8_t *d_native, float *d_scales, float *d_rot_out,
                          hipStream_t s);
+size_t encode_lds_bytes(int dim);
 hipError_t launch_move_lane(uint8_t *d_native, float *d_scales, const Geometry &g, size_t src, size_t dst,
                             hipStream_t s);
 
@@ -119,10 +121,11 @@ hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, cons
 // Gathers each query's candidate segments (n_seg of them, seg_stride allocated), sorts, and either
 // emits the k_eff best (tau_out == nullptr; a query that did not fit is flagged in overflow) or, for a
 // sampling level, writes the order key of the k_floor-th best as the query's next floor to
-// tau_out[(q / tau_stride_q) * kQTile + q % tau_stride_q].
+// tau_out[(q / tau_stride_q) * kQTile + q % tau_stride_q] (keep_floor: a level that gathers fewer than k_eff
+// candidates leaves the floor already there in place instead of opening it).
 hipError_t launch_final(const uint64_t *cand, const uint32_t *cand_cnt, uint32_t n_seg, uint32_t seg_stride,
                         int k_eff, int k_floor, int nq, float *out_scores, int64_t *out_idx, uint32_t *overflow,
-                        int *tau_out, int tau_stride_q, hipStream_t s);
+                        int *tau_out, int tau_stride_q, int keep_floor, hipStream_t s);
 hipError_t launch_fill_i32(int *p, int v, size_t n, hipStream_t s);
 hipError_t launch_probe(const void *src, void *dst, size_t bytes, int copy, uint32_t *sink, hipStream_t s);
 hipError_t launch_probe_mfma(int device, int iters, uint32_t *sink, double *ops, hipStream_t s);
@@ -145,7 +148,8 @@ struct tv_index {
     float cs = 1.0f;
 
     hipStream_t stream = nullptr;
-    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    hipEvent_t ev_start[tv::kTimedLaunches] = {}, ev_stop[tv::kTimedLaunches] = {};
+    bool events_ready = false;
     float *d_signs = nullptr;
     uint32_t *d_perms = nullptr;
     float *d_centroids = nullptr;

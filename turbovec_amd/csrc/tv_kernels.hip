@@ -927,7 +927,7 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
                                                uint32_t seg_stride, int k_eff, int k_floor,
                                                float *__restrict__ out_scores, int64_t *__restrict__ out_idx,
                                                uint32_t *__restrict__ overflow, int *__restrict__ tau_out,
-                                               int tau_stride_q) {
+                                               int tau_stride_q, int keep_floor) {
     __shared__ uint64_t keys[kFinalCap];
     __shared__ uint32_t wave_sum[kFinalThreads / 64];
     __shared__ uint32_t any_full, long_n;
@@ -965,7 +965,10 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
         if (redo) return;
     }
     if (sampling && total < uint32_t(k_eff)) {
-        if (t == 0) *tau_slot = kTauInit;  // too few allowed slots sampled: the floor stays open
+        // Too few allowed slots reached the floor in this sample.  The floor of the level before
+        // (k_floor scanned slots reach it) is still a valid lower bound: it stays.  Only the
+        // first level, which reads the standing array of open floors, has none to keep.
+        if (t == 0 && !keep_floor) *tau_slot = kTauInit;
         return;
     }
     // gather (a sampling level may keep any subset: dropping what does not fit only loosens the floor).
@@ -1376,10 +1379,10 @@ hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, cons
 
 hipError_t launch_final(const uint64_t *cand, const uint32_t *cand_cnt, uint32_t n_seg, uint32_t seg_stride,
                         int k_eff, int k_floor, int nq, float *out_scores, int64_t *out_idx, uint32_t *overflow,
-                        int *tau_out, int tau_stride_q, hipStream_t s) {
+                        int *tau_out, int tau_stride_q, int keep_floor, hipStream_t s) {
     if (nq == 0 || k_eff == 0) return hipSuccess;
     hipLaunchKernelGGL(k_final, dim3(nq), dim3(kFinalThreads), 0, s, cand, cand_cnt, n_seg, seg_stride, k_eff, k_floor,
-                       out_scores, out_idx, overflow, tau_out, tau_stride_q);
+                       out_scores, out_idx, overflow, tau_out, tau_stride_q, keep_floor);
     return hipGetLastError();
 }
 

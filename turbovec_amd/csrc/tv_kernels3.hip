@@ -36,7 +36,7 @@ constexpr int kWideRing = 5;         // LDS slots of one slice each; kWideRing -
 // like a load.  Uniform bases live in scalar registers: the kernel has no vector register to spare.
 __device__ __forceinline__ void dma16_to_lds(uint32_t lds_addr, const void *sbase, uint32_t lane16) {
     const uint32_t u = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_addr)));
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(u), "v"(lane16), "s"(sbase) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(u), "v"(lane16), "s"(sbase) : "memory", "m0");
 }
 
 // 16 bytes per lane from uniform base + 16 * lane into registers, invisible to the compiler's
@@ -109,7 +109,11 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
         sq[q].tau = tau;
         sq[q].cnt = 0u;
         const float inf = __int_as_float(0x7f800000);
-        const bool bounded = tau > 0.0f && tau < inf && qs > 0.0f && qs < inf && fabsf(qb) < inf;
+        // The bound's error analysis assumes normal floats throughout: outside 1e-30 .. 1e30
+        // (subnormal floors round coarsely; tau / qs may overflow and still be met by a huge row
+        // scale) there is no bound and every tile is scored.
+        const bool bounded = tau >= 1e-30f && tau <= 1e30f && qs >= 1e-30f && qs <= 1e30f && fabsf(qb) <= 1e30f &&
+                             tau / qs < inf;
         const float rb = qb / qs;
         sq[q].ta = !act ? inf : bounded ? (tau / qs) * (1.0f - 1e-5f) : -inf;
         sq[q].tb = act && bounded ? rb + 1e-5f * fabsf(rb) + 2.0f : 0.0f;
@@ -249,15 +253,20 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
             }
             // row scales (NaN where not allowed, and for a block slot left empty: its stale
             // operands then score nothing); their maximum over the allowed rows feeds the
-            // accumulator bound, and a block with a negative or non-finite one (no encoder
+            // accumulator bound, and a block with a negative, huge or non-finite one (no encoder
             // writes such) is always scored
             if (lane < 32) s_vs[(wave * BLK + k) * 32 + lane] = sc;
             float vmax = ok ? sc : 0.0f;
-            const bool odd = ok && !(sc >= 0.0f && sc < __int_as_float(0x7f800000));
+            const bool odd = ok && !(sc >= 0.0f && sc <= 1e30f);
 #pragma unroll
             for (int d = 16; d >= 1; d >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, d));
-            odd_block[k] = __any(odd);
-            inv_vmax[k] = __builtin_amdgcn_readfirstlane(__float_as_int(1.0f / vmax));
+            // A largest row scale below 1e-30 (a foreign snapshot may hold subnormal scales; no
+            // encoder writes them) has a reciprocal that overflows or rounds coarsely: such a
+            // block is always scored too.  All scales zero: every score is zero, below any
+            // positive floor, and the infinite bound is right.
+            const float inv = 1.0f / vmax;
+            odd_block[k] = __any(odd) || (vmax > 0.0f && vmax < 1e-30f);
+            inv_vmax[k] = __builtin_amdgcn_readfirstlane(__float_as_int(inv));
         });
         if (!__syncthreads_or(has ? 1 : 0)) break;
 

@@ -14,8 +14,11 @@ Snapshots: `to_bytes` / `from_bytes` / `write` / `load` produce and read the
 reference's image bytes (turbovec/src/io_v7.rs; lib.rs:2167 to_bytes, id_map.rs:971)
 through tv_index_to_bytes / tv_index_from_bytes.
 
+Pickling, `copy` and `deepcopy` go through `from_bytes(to_bytes())`, as the
+reference's bindings reduce them (turbovec-python/src/lib.rs `__reduce__`).
+
 Not mirrored (outside the search path): sync (the incremental container),
-calibrate on a populated index (re-encoding stored rows), pickling.
+calibrate on a populated index (re-encoding stored rows).
 """
 import os
 import threading
