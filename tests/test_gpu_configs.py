@@ -1,4 +1,4 @@
-"""Benchmark configurations 3, 4 and 5 at their full sizes, through size-independent
+"""Benchmark configurations 2, 3, 4 and 5 at their full sizes and prescribed batches, through size-independent
 properties (the oracle cannot finish these in seconds):
 
   * the rows returned equal an independent ranking of the per-slot scores the
@@ -64,36 +64,75 @@ def merged(parts, k):
 
 
 def test_config3_10m_1536_2bit_k100(T):
-    dim, bits, n, k = 1536, 2, 10_000_000, 100
+    """Configuration 3 as stated: 10M x 1536 2-bit, added in 100k chunks, k=100, batches of 1 and 1024."""
+    dim, bits, n, k, nq = 1536, 2, 10_000_000, 100, 1024
     gen = torch.Generator(device="cuda"); gen.manual_seed(0)
     ix = T.NativeIndex(dim, bits)
     add_generated(ix, n, dim, lambda c0, m: unit_rows(gen, m, dim))
     assert len(ix) == n
     qgen = torch.Generator(device="cuda"); qgen.manual_seed(1)
-    q = unit_rows(qgen, 64, dim).cpu().numpy()
+    q = unit_rows(qgen, nq, dim).cpu().numpy()
     s, i = ix.search(q, k)
-    assert s.shape == (64, k) and np.all(np.diff(s.astype(np.float64), axis=1) <= 0)
+    assert s.shape == (nq, k) and np.all(np.diff(s.astype(np.float64), axis=1) <= 0)
     assert all(len(set(r.tolist())) == k for r in i)
-    _acc, raw = ix.debug_scan(q[:2])
-    for r in range(2):
+    assert ix.overflow_redos() == 0                     # Gaussian rows never leave the sampled path
+    # rows 0, 1 and two from the far end of the batch against an independent ranking of dumped scores
+    probe = np.array([0, 1, 517, 1023])
+    _acc, raw = ix.debug_scan(q[probe])
+    for r, qi in enumerate(probe):
         order = independent_topk(raw[r], k)
-        assert i[r].tolist() == order.tolist() and bits_equal(s[r], raw[r][order])
-    s1, i1 = ix.search(q[3:4], k)                       # batch 1 == its row of the batch
-    assert np.array_equal(i1[0], i[3]) and bits_equal(s1[0], s[3])
+        assert i[qi].tolist() == order.tolist() and bits_equal(s[qi], raw[r][order])
+    for qi in (3, 1000):                                # batch 1 == its row of the batch
+        s1, i1 = ix.search(q[qi:qi + 1], k)
+        assert np.array_equal(i1[0], i[qi]) and bits_equal(s1[0], s[qi])
+    s64, i64 = ix.search(q[100:164], k)                 # and a 64-query batch its 64 rows
+    assert np.array_equal(i64, i[100:164]) and bits_equal(s64, s[100:164])
     ix.set_path(1)                                      # exact select path
     s2, i2 = ix.search(q[:8], k)
     ix.set_path(0)
     assert np.array_equal(i2, i[:8]) and bits_equal(s2, s[:8])
+    assert ix.overflow_redos() == 0
+    ix.close()
+
+
+def test_config2_1m_1536_4bit_encoded_rows(T):
+    """Configuration 2 as stated: 1M encoded Gaussian rows (seed 0), batches of 1, 64 and 1024, k=10."""
+    dim, bits, n, k = 1536, 4, 1_000_000, 10
+    gen = torch.Generator(device="cuda"); gen.manual_seed(0)
+    ix = T.NativeIndex(dim, bits)
+    add_generated(ix, n, dim, lambda c0, m: unit_rows(gen, m, dim))
+    qgen = torch.Generator(device="cuda"); qgen.manual_seed(1)
+    q = unit_rows(qgen, 1024, dim).cpu().numpy()
+    s, i = ix.search(q, k)
+    assert s.shape == (1024, k) and ix.queries_per_launch() == 1024    # the all-queries-per-pass kernel
+    probe = np.array([0, 1, 2, 640, 1023])
+    _acc, raw = ix.debug_scan(q[probe])
+    for r, qi in enumerate(probe):
+        order = independent_topk(raw[r], k)
+        assert i[qi].tolist() == order.tolist() and bits_equal(s[qi], raw[r][order])
+    s64, i64 = ix.search(q[64:128], k)
+    assert np.array_equal(i64, i[64:128]) and bits_equal(s64, s[64:128])
+    for qi in (5, 999):
+        s1, i1 = ix.search(q[qi:qi + 1], k)
+        assert np.array_equal(i1[0], i[qi]) and bits_equal(s1[0], s[qi])
+    for path in (1, 4):                                 # exact lists; tile-group kernel
+        ix.set_path(path)
+        s2, i2 = ix.search(q[:160], k)
+        ix.set_path(0)
+        assert np.array_equal(i2, i[:160]) and bits_equal(s2, s[:160])
+    assert ix.overflow_redos() == 0
     ix.close()
 
 
 def test_config4_idmap_2m_3072_allowlists():
+    """Configuration 4 as stated: IdMapIndex 2M x 3072 4-bit, 1024 queries, k=10, the three allowlists."""
     from turbovec_amd import index as api
-    dim, n = 3072, 2_000_000
+    dim, n, nq = 3072, 2_000_000, 1024
     gen = torch.Generator(device="cuda"); gen.manual_seed(0)
     idx = api.IdMapIndex(dim, 4)
     rng = np.random.default_rng(0)
     ids = (rng.permutation(n).astype(np.uint64) * np.uint64(2654435761) + np.uint64(12345))   # unique
+    id_to_slot = {int(v): j for j, v in enumerate(ids.tolist())}
     planted = None
     for c0 in range(0, n, 100_000):
         v = unit_rows(gen, 100_000, dim).cpu().numpy()
@@ -101,36 +140,64 @@ def test_config4_idmap_2m_3072_allowlists():
             planted = v[:64].copy()
         idx.add_with_ids(v, ids[c0:c0 + 100_000])
     assert len(idx) == n
+    native = idx._inner._ix
     noise = np.random.default_rng(1).standard_normal(planted.shape).astype(np.float32) * np.float32(0.05 / np.sqrt(dim))
-    q = planted + noise
+    q = np.concatenate([planted + noise, np.random.default_rng(2).standard_normal((nq - 64, dim)).astype(np.float32)])
     q /= np.linalg.norm(q, axis=1, keepdims=True)
     s, g = idx.search(q, 10)
-    assert s.shape == (64, 10) and (g[:, 0] == ids[:64]).all()           # each query finds its source row
-    # (a) 1 % of the ids, uniformly at random, the planted rows' ids included for half the queries
+    assert native.queries_per_launch() == nq                              # one pass of the wide kernel
+    assert s.shape == (nq, 10) and (g[:64, 0] == ids[:64]).all()          # each planted query finds its source row
+    probe = np.array([0, 63, 64, 700, 1023])
+    _acc, raw = native.debug_scan(q[probe])
+
+    def check_rows(scores, got_ids, k, allowed_slots=None):
+        allowed = None
+        if allowed_slots is not None:
+            allowed = np.zeros(n, bool)
+            allowed[allowed_slots] = True
+        for r, qi in enumerate(probe):
+            order = independent_topk(raw[r], k, allowed=allowed)
+            if allowed is not None:
+                order = order[:int(allowed.sum())]
+            assert [id_to_slot[int(x)] for x in got_ids[qi]] == order.tolist()
+            assert bits_equal(scores[qi], raw[r][order])
+
+    check_rows(s, g, 10)
+    # (a) 1 % of the ids, uniformly at random, the planted rows' ids included for half of the planted queries
     allow_a = np.concatenate([ids[rng.choice(n, n // 100, replace=False)], ids[:32]])
     sa, ga = idx.search(q, 10, allowlist=allow_a)
     aset = set(allow_a.tolist())
-    assert sa.shape == (64, 10) and all(x in aset for x in ga.ravel().tolist())
+    assert sa.shape == (nq, 10) and all(x in aset for x in ga.ravel().tolist())
     assert (ga[:32, 0] == ids[:32]).all()
     assert np.all(sa[32:, 0] <= s[32:, 0])
+    check_rows(sa, ga, 10, np.array(sorted({id_to_slot[int(x)] for x in allow_a.tolist()})))
     # (b) a contiguous 5 % run of insertion order
     allow_b = ids[1_000_000:1_100_000]
     sb, gb = idx.search(q, 10, allowlist=allow_b)
     bset = set(allow_b.tolist())
-    assert sb.shape == (64, 10) and all(x in bset for x in gb.ravel().tolist())
-    # filtered top-k of (a) and (b) both equal the full ranking restricted to the filter where they meet it
-    for r in range(64):
+    assert sb.shape == (nq, 10) and all(x in bset for x in gb.ravel().tolist())
+    check_rows(sb, gb, 10, np.arange(1_000_000, 1_100_000))
+    # filtered top-k of (a) equals the full ranking restricted to the filter where they meet it
+    for r in range(nq):
         in_a = [x for x in g[r].tolist() if x in aset]
         assert ga[r].tolist()[:len(in_a)] == in_a
     # (c) sixteen ids, fewer than k=100: rows of exactly sixteen, the same set for every query
-    allow_c = ids[[7, 99, 1234, 50_000, 123_456, 500_000, 999_999, 1_000_000, 1_000_001, 1_500_000,
-                   1_999_999, 31, 32, 33, 64, 0]]
+    c_slots = np.array([7, 99, 1234, 50_000, 123_456, 500_000, 999_999, 1_000_000, 1_000_001, 1_500_000,
+                        1_999_999, 31, 32, 33, 64, 0])
+    allow_c = ids[c_slots]
     sc, gc = idx.search(q, 100, allowlist=allow_c)
-    assert sc.shape == (64, 16) and all(set(r.tolist()) == set(allow_c.tolist()) for r in gc)
+    assert sc.shape == (nq, 16) and all(set(r.tolist()) == set(allow_c.tolist()) for r in gc)
     assert np.all(np.diff(sc.astype(np.float64), axis=1) <= 0)
+    check_rows(sc, gc, 100, np.sort(c_slots))
     sc10, gc10 = idx.search(q, 10, allowlist=allow_c)
-    assert sc10.shape == (64, 10) and np.array_equal(gc10, gc[:, :10]) and bits_equal(sc10, sc[:, :10])
+    assert sc10.shape == (nq, 10) and np.array_equal(gc10, gc[:, :10]) and bits_equal(sc10, sc[:, :10])
     assert (gc[0, 0] == ids[0])                                           # slot 0 is query 0's source
+    # the tile-group kernel gives the same rows for the filtered batch
+    native.set_path(4)
+    sa2, ga2 = idx.search(q[:200], 10, allowlist=allow_a)
+    native.set_path(0)
+    assert np.array_equal(ga2, ga[:200]) and bits_equal(sa2, sa[:200])
+    assert native.overflow_redos() == 0
 
 
 def test_config5_10m_1536_clustered_mask_and_churn(T):
@@ -195,4 +262,7 @@ def test_config5_10m_1536_clustered_mask_and_churn(T):
     assert i4[0].tolist() == order.tolist() and bits_equal(s4[0], raw[0][order])
     order = independent_topk(raw[0], k)
     assert i3[0].tolist() == order.tolist() and bits_equal(s3[0], raw[0][order])
+    # clustered rows, queries next to database rows: results stay exact whatever the count; the
+    # sampled path is expected to hold (a redo is the exact path's time, not a wrong answer)
+    assert ix.overflow_redos() == 0
     ix.close()

@@ -407,8 +407,9 @@ def test_handed_over_tables_are_used(T, oracle):
 
 
 # ---- benchmark-sized inputs: size-independent properties ----
-def test_config2_scale_properties(T):
-    """1M x 1536 4-bit (benchmark config 2) with synthetic codes: the top-k the
+def test_random_codes_scale_properties(T):
+    """1M x 1536 4-bit of uniform random code bytes and scales (configuration 2 itself, on encoded
+    Gaussian rows, is in test_gpu_configs.py): the top-k the
     search returns equals an independent ranking of the dumped per-slot scores;
     batches of 1, 64 and 1024 agree row by row; top-10 is a prefix of top-32."""
     dim, bits, n = 1536, 4, 1_000_000

@@ -150,6 +150,8 @@ __global__ __launch_bounds__(256) void k_encode(EncodeArgs a) {
 
 // A and B, one float row each; codes and the f64 products overlay A.  128 KiB at the largest
 // row the index accepts (16384 dimensions), inside the 160 KiB a workgroup may have.
+static_assert(size_t(2) * 16384 * sizeof(float) + 4 * sizeof(double) <= 160 * 1024,
+              "the longest row the index accepts (lib.rs:101 MAX_DIM) must fit a workgroup's LDS");
 size_t encode_lds_bytes(int dim) { return size_t(2) * size_t(dim) * sizeof(float) + 4 * sizeof(double); }
 
 hipError_t launch_encode(const float *d_vecs, size_t n_new, size_t old_n, const float *d_signs,
