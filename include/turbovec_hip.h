@@ -150,6 +150,24 @@ int tv_search_dev(tv_index *ix, const float *d_queries, size_t nq, size_t k,
                   const uint64_t *d_mask_words, size_t n_allowed,
                   float *d_out_scores, int64_t *d_out_indices, size_t *out_k_eff);
 
+/* tv_search_dev for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments, results and status codes as tv_search_dev, but everything the search carves
+ * -- rotated queries, tables, candidate segments, the exact path's lists -- comes out of a
+ * fixed array in the library's device image (tv_noalloc_scratch_bytes() bytes, 64 MiB, held by
+ * every GPU the library runs on until the process ends), and the call makes no hipMalloc,
+ * hipFree, event or stream creation.  A search whose worst case does not fit (at 1536
+ * dimensions, 4-bit: more than about 400 queries per call; k > 32 on an index of millions of
+ * rows, whose exact fallback ranks dense score rows) is refused with TV_ERR_BAD_ARGUMENT and
+ * tv_last_error() names the bytes needed; nothing is written then.  All calls on one GPU share
+ * the array: within a process they are serialised by the library; the array keeps the previous
+ * call's bytes and every search overwrites what it reads.  Scan timings (tv_last_scan_ms) are
+ * not taken on this path. */
+int tv_search_dev_noalloc(tv_index *ix, const float *d_queries, size_t nq, size_t k,
+                          const uint64_t *d_mask_words, size_t n_allowed,
+                          float *d_out_scores, int64_t *d_out_indices, size_t *out_k_eff);
+size_t tv_noalloc_scratch_bytes(void);
+
 /* ---- host-only derivations (no GPU touched) ------------------------------- */
 
 /* The tables tv_index_create derives: Rotation::new (rotation.rs:141-187;

@@ -32,7 +32,7 @@ EXPORTS = [
     "tv_debug_prepare", "tv_last_scan_ms", "tv_debug_queries_per_launch", "tv_index_device_ptrs", "tv_host_rotation_tables", "tv_host_codebook",
     "tv_debug_stream_probe", "tv_debug_mfma_probe", "tv_debug_set_path", "tv_debug_overflow_redos",
     "tv_host_snapshot_len", "tv_host_snapshot_compose", "tv_host_snapshot_info", "tv_host_snapshot_extract",
-    "tv_index_to_bytes", "tv_index_from_bytes",
+    "tv_index_to_bytes", "tv_index_from_bytes", "tv_search_dev_noalloc", "tv_noalloc_scratch_bytes",
 ]
 
 _lib = None
@@ -88,6 +88,9 @@ def lib():
     L.tv_pack_mask.argtypes = [vp, sz, vp, C.POINTER(sz)]
     L.tv_search.argtypes = [vp, vp, sz, sz, vp, sz, vp, vp, C.POINTER(sz)]
     L.tv_search_dev.argtypes = [vp, vp, sz, sz, vp, sz, vp, vp, C.POINTER(sz)]
+    L.tv_search_dev_noalloc.argtypes = [vp, vp, sz, sz, vp, sz, vp, vp, C.POINTER(sz)]
+    L.tv_noalloc_scratch_bytes.restype = sz
+    L.tv_noalloc_scratch_bytes.argtypes = []
     L.tv_debug_scan.argtypes = [vp, vp, sz, vp, vp]
     L.tv_debug_prepare.argtypes = [vp, vp, sz, vp, vp, vp]
     L.tv_last_scan_ms.argtypes = [vp, C.POINTER(C.c_float), C.POINTER(i32)]
@@ -257,6 +260,13 @@ class NativeIndex:
         k_eff = C.c_size_t(0)
         check(lib().tv_search_dev(self.h, d_queries_ptr, nq, k, d_mask_ptr, n_allowed, d_out_scores_ptr,
                                   d_out_idx_ptr, C.byref(k_eff)))
+        return k_eff.value
+
+    def search_dev_noalloc(self, d_queries_ptr, nq, k, d_out_scores_ptr, d_out_idx_ptr, d_mask_ptr=None, n_allowed=0):
+        """tv_search_dev on the library's fixed scratch array: no device allocation inside the call."""
+        k_eff = C.c_size_t(0)
+        check(lib().tv_search_dev_noalloc(self.h, d_queries_ptr, nq, k, d_mask_ptr, n_allowed, d_out_scores_ptr,
+                                          d_out_idx_ptr, C.byref(k_eff)))
         return k_eff.value
 
     def debug_scan(self, queries):

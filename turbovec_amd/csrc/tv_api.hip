@@ -44,8 +44,43 @@ struct Arena {
     }
 };
 
+// ---- the scratch buffer of tv_search_dev_noalloc ---------------------------------------------
+// One array per GPU, in the library's device image: every device the library runs on holds
+// kScratchBytes of it from the moment the image is loaded there until the process ends.  In host
+// code the array's name is only a handle for hipGetSymbolAddress; each device's copy has an
+// address of its own, looked up once per device and kept in g_scratch.
+constexpr size_t kScratchBytes = size_t(64) << 20;
+static __device__ __align__(256) uint8_t scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+struct DeviceScratch {
+    void *ptr = nullptr;     // device address of `scratch` on this device
+    std::mutex in_use;       // calls on one device share the array: one at a time within the process
+};
+DeviceScratch g_scratch[kMaxDevices];
+std::mutex g_scratch_setup;
+
+// Device `device` must be current.
+int scratch_address(int device, void **out) {
+    if (device < 0 || device >= kMaxDevices) { g_last_error = "device ordinal beyond the scratch table"; return TV_ERR_NO_DEVICE; }
+    std::lock_guard<std::mutex> lock(g_scratch_setup);
+    if (!g_scratch[device].ptr) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return fail_hip(e, "hipGetSymbolAddress(scratch)");
+        g_scratch[device].ptr = p;
+    }
+    *out = g_scratch[device].ptr;
+    return TV_OK;
+}
+
 int ensure_workspace(tv_index *ix, size_t bytes) {
     if (bytes <= ix->ws_bytes) return TV_OK;
+    if (ix->ws_fixed) {   // the caller lent a buffer of fixed size: never replaced
+        g_last_error = "search needs " + std::to_string(bytes) + " bytes of scratch, the fixed buffer holds " +
+                       std::to_string(ix->ws_bytes);
+        return TV_ERR_BAD_ARGUMENT;
+    }
     if (ix->ws) { TV_HIP(hipFree(ix->ws)); ix->ws = nullptr; ix->ws_bytes = 0; }
     bytes = round_up(bytes + bytes / 4, size_t(1) << 20);
     TV_HIP(hipMalloc(&ix->ws, bytes));
@@ -222,6 +257,49 @@ int ensure_events(tv_index *ix) {
     return TV_OK;
 }
 
+// Workspace bytes one chunk of cq queries needs on the exact path (search_robust) ...
+size_t robust_need(const tv_index *ix, size_t cq, size_t k_eff) {
+    const tv::Geometry &g = ix->geo;
+    const bool mode_p = effective_mode(ix) == TV_SCORE_P;
+    const bool lists = k_eff <= size_t(tv::kMaxListK);
+    const int kl = lists ? int(k_eff) : 1;
+    const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_tile_queries(g.nch, kl));
+    const size_t n_tiles = (cq + tile_q - 1) / tile_q;
+    const int grid = tv::scan_grid_blocks(ix->device, mode_p, g.nch, kl, int(tile_q));
+    const size_t total_threads = size_t(grid) * tv::kScanThreads;
+    size_t need = prepare_bytes(ix, cq) + round_up(n_tiles * tv::kQTile * 4, 256);
+    if (lists) need += 2 * round_up(k_eff * total_threads * 4, 256) + round_up(total_threads * 4, 256);
+    else need += round_up(size_t(tv::kQTile) * ix->n * 4, 256) + round_up(tv::select_tmp_keys(k_eff) * 8 * tv::kQTile, 256) +
+                 round_up(size_t(tv::kQTile) * 4096 * 4, 256);
+    return need + 65536;
+}
+
+// ... and on the sampled path (search_device): prepared queries, floors, candidate segments.
+struct SampledPlan {
+    size_t tile_q, n_tiles, cq_pad, seg_stride, need;
+    bool wide;
+    int grid;
+};
+SampledPlan sampled_plan(const tv_index *ix, size_t cq) {
+    const tv::Geometry &g = ix->geo;
+    const bool mode_p = effective_mode(ix) == TV_SCORE_P;
+    SampledPlan p;
+    p.tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_append_queries(g.nch));
+    p.n_tiles = (cq + p.tile_q - 1) / p.tile_q;
+    p.cq_pad = p.n_tiles * p.tile_q;
+    // large chunks of high-dimensional queries take the wide kernel: all of them in one pass per level
+    const int wide_min = tv::wide_min_queries(g.nch);
+    p.wide = mode_p && !ix->no_batched && !ix->no_wide && wide_min > 0 && cq >= size_t(wide_min);
+    p.grid = p.wide ? tv::wide_grid_blocks(ix->device)
+           : mode_p ? tv::scan_grid_blocks(ix->device, mode_p, g.nch, 0, int(p.tile_q))
+                    : tv::lut_append_grid(ix->device, g.nch);
+    p.seg_stride = size_t(p.grid);
+    p.need = prepare_bytes(ix, cq) + round_up(p.n_tiles * tv::kQTile * 4, 256) +
+             round_up(p.cq_pad * p.seg_stride * tv::kSegCap * 8, 256) + round_up(p.cq_pad * p.seg_stride * 4, 256) +
+             round_up(p.cq_pad * 4, 256) + 65536;
+    return p;
+}
+
 // Full-range search without sampling: per-lane lists with shared thresholds for
 // k <= 32, dense scores + radix select beyond.  Always exact; used for the
 // queries whose candidate buffer overflowed and for very large k.
@@ -240,11 +318,7 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
         const size_t n_tiles = (cq + tile_q - 1) / tile_q;
         const int grid = tv::scan_grid_blocks(ix->device, mode_p, g.nch, kl, int(tile_q));
         const size_t total_threads = size_t(grid) * tv::kScanThreads;
-        size_t need = prepare_bytes(ix, cq) + round_up(n_tiles * tv::kQTile * 4, 256);
-        if (lists) need += 2 * round_up(k_eff * total_threads * 4, 256) + round_up(total_threads * 4, 256);
-        else need += round_up(size_t(tv::kQTile) * n * 4, 256) + round_up(tv::select_tmp_keys(k_eff) * 8 * tv::kQTile, 256) +
-                     round_up(size_t(tv::kQTile) * 4096 * 4, 256);
-        rc = ensure_workspace(ix, need + 65536);
+        rc = ensure_workspace(ix, robust_need(ix, cq, k_eff));
         if (rc != TV_OK) return rc;
         Arena ar;
         ar.base = static_cast<uint8_t *>(ix->ws);
@@ -316,22 +390,29 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
 // candidates per query (the floor is the k_floor-th best of the level before,
 // so a level `ratio` times larger keeps about ratio * k_floor).  The sampling
 // levels together read about 1/ratio of the index.
-std::vector<uint32_t> sampling_steps(size_t n_blocks, size_t k_floor) {
+struct SamplingSteps {
+    static constexpr int kMax = 32;   // levels grow at least fourfold: 2^31 slots need 16 at most
+    uint32_t step[kMax];
+    size_t count = 0;
+    size_t size() const { return count; }
+    uint32_t operator[](size_t i) const { return step[i]; }
+};
+SamplingSteps sampling_steps(size_t n_blocks, size_t k_floor) {
     const double n_slots = double(n_blocks * tv::kVecBlock);
     const double first = double(std::max<size_t>(1024, 8 * k_floor));
-    std::vector<uint32_t> steps;
+    SamplingSteps steps;
     if (n_slots > 2.0 * first) {
         const double max_ratio = std::max(4.0, double(tv::kFinalCap / 2) / double(k_floor));
         const int levels = std::max(1, int(std::ceil(std::log(n_slots / first) / std::log(max_ratio))));
         const double ratio = std::pow(n_slots / first, 1.0 / double(levels));
         double sample = first;
-        for (int lv = 0; lv < levels; ++lv, sample *= ratio) {
+        for (int lv = 0; lv < levels && steps.count + 1 < size_t(SamplingSteps::kMax); ++lv, sample *= ratio) {
             const size_t sample_blocks = std::max<size_t>(1, size_t(sample) / tv::kVecBlock);
             const size_t step = n_blocks / sample_blocks;
-            if (step > 1 && (steps.empty() || step < steps.back())) steps.push_back(uint32_t(step));
+            if (step > 1 && (steps.count == 0 || step < steps.step[steps.count - 1])) steps.step[steps.count++] = uint32_t(step);
         }
     }
-    steps.push_back(1);
+    steps.step[steps.count++] = 1;
     return steps;
 }
 
@@ -357,33 +438,26 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
     const int mode = effective_mode(ix);
     if (mode == TV_SCORE_P && g.bits != 4) { g_last_error = "score mode P needs 4-bit codes"; return TV_ERR_BAD_ARGUMENT; }
     const bool mode_p = mode == TV_SCORE_P;
-    int rc = ensure_events(ix);
+    // a search on a lent, fixed workspace (tv_search_dev_noalloc) creates nothing, event pool included
+    const bool timing = !ix->ws_fixed;
+    int rc = timing ? ensure_events(ix) : TV_OK;
     if (rc != TV_OK) return rc;
     if (k_eff > size_t(tv::kMaxSampledK) || ix->force_robust)
-        return search_robust(ix, d_queries, nq, k_eff, d_mask, d_out_scores, d_out_idx, true);
+        return search_robust(ix, d_queries, nq, k_eff, d_mask, d_out_scores, d_out_idx, timing);
 
     const size_t n_blocks = (n + tv::kVecBlock - 1) / tv::kVecBlock;
     // sampling levels take the k_floor-th best as the floor: a deeper order statistic is steadier
     const size_t k_floor = std::max<size_t>(k_eff, 16);
-    const std::vector<uint32_t> steps = sampling_steps(n_blocks, k_floor);
-    std::vector<uint32_t> h_over;
+    const SamplingSteps steps = sampling_steps(n_blocks, k_floor);
+    uint32_t *h_over = ix->h_flags;   // pinned, one flag per query of a chunk
 
     for (size_t q0 = 0; q0 < nq; q0 += kChunkQueries) {
         const size_t cq = std::min(kChunkQueries, nq - q0);
-        const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_append_queries(g.nch));
-        const size_t n_tiles = (cq + tile_q - 1) / tile_q;
-        const size_t cq_pad = n_tiles * tile_q;
-        // large chunks of high-dimensional queries take the wide kernel: all of them in one pass per level
-        const int wide_min = tv::wide_min_queries(g.nch);
-        const bool wide = mode_p && !ix->no_batched && !ix->no_wide && wide_min > 0 && cq >= size_t(wide_min);
-        const int grid = wide ? tv::wide_grid_blocks(ix->device)
-                       : mode_p ? tv::scan_grid_blocks(ix->device, mode_p, g.nch, 0, int(tile_q))
-                                : tv::lut_append_grid(ix->device, g.nch);
-        const size_t seg_stride = size_t(grid);
-        size_t need = prepare_bytes(ix, cq) + round_up(n_tiles * tv::kQTile * 4, 256) +
-                      round_up(cq_pad * seg_stride * tv::kSegCap * 8, 256) + round_up(cq_pad * seg_stride * 4, 256) +
-                      round_up(cq_pad * 4, 256);
-        rc = ensure_workspace(ix, need + 65536);
+        const SampledPlan plan = sampled_plan(ix, cq);
+        const size_t tile_q = plan.tile_q, n_tiles = plan.n_tiles, cq_pad = plan.cq_pad, seg_stride = plan.seg_stride;
+        const bool wide = plan.wide;
+        const int grid = plan.grid;
+        rc = ensure_workspace(ix, plan.need);
         if (rc != TV_OK) return rc;
         Arena ar;
         ar.base = static_cast<uint8_t *>(ix->ws);
@@ -424,7 +498,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
                 a.cand = d_cand + t * tile_q * seg_stride * tv::kSegCap;
                 a.cand_cnt = d_cnt + t * tile_q * seg_stride;
                 a.seg_stride = uint32_t(seg_stride);
-                const bool timed = last && int(launch_no) < kMaxTimedTiles;
+                const bool timed = timing && last && int(launch_no) < kMaxTimedTiles;
                 if (timed) TV_HIP(hipEventRecord(ix->ev_start[launch_no], ix->stream));
                 if (wide) {
                     n_seg = grid;
@@ -439,13 +513,12 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
                 }
                 if (timed) TV_HIP(hipEventRecord(ix->ev_stop[launch_no], ix->stream));
             }
-            if (last) n_timed = std::min<size_t>(launch_no, size_t(kMaxTimedTiles));
+            if (last && timing) n_timed = std::min<size_t>(launch_no, size_t(kMaxTimedTiles));
             TV_HIP(tv::launch_final(d_cand, d_cnt, uint32_t(n_seg), uint32_t(seg_stride), int(k_eff), int(k_floor),
                                     int(cq), d_out_scores + q0 * k_eff, d_out_idx + q0 * k_eff, d_over,
                                     last ? nullptr : d_tau, int(tile_q), lv > 0 ? 1 : 0, ix->stream));
         }
-        h_over.resize(cq);
-        TV_HIP(hipMemcpyAsync(h_over.data(), d_over, cq * sizeof(uint32_t), hipMemcpyDeviceToHost, ix->stream));
+        TV_HIP(hipMemcpyAsync(h_over, d_over, cq * sizeof(uint32_t), hipMemcpyDeviceToHost, ix->stream));
         TV_HIP(hipStreamSynchronize(ix->stream));
         for (size_t t = 0; t < n_timed; ++t) {
             float ms = 0.0f;
@@ -525,6 +598,12 @@ int tv_index_create(int dim, int bits, int device, tv_index **out) {
             rc = TV_ERR_HIP;
             break;
         }
+        if (hipHostMalloc(reinterpret_cast<void **>(&ix->h_flags), kChunkQueries * sizeof(uint32_t), hipHostMallocDefault) != hipSuccess) {
+            rc = TV_ERR_HIP;
+            break;
+        }
+        rc = scratch_address(device, &ix->scratch);
+        if (rc != TV_OK) break;
         // floors of a search's first sampling level: the order key of -inf for every query, written once
         if (tv::launch_fill_i32(ix->d_tau_open, int(0x807fffffu), kTauOpenInts, ix->stream) != hipSuccess ||
             hipStreamSynchronize(ix->stream) != hipSuccess) {
@@ -549,6 +628,7 @@ int tv_index_destroy(tv_index *ix) {
     void *ptrs[] = {ix->d_signs, ix->d_perms, ix->d_centroids, ix->d_tq_shift, ix->d_tq_scale,
                     ix->d_codes, ix->d_scales, ix->ws, ix->io, ix->d_tau_open};
     for (void *p : ptrs) if (p) (void)hipFree(p);
+    if (ix->h_flags) (void)hipHostFree(ix->h_flags);
     if (ix->events_ready)
         for (int i = 0; i < tv::kTimedLaunches; ++i) {
             (void)hipEventDestroy(ix->ev_start[i]);
@@ -869,6 +949,43 @@ int tv_search_dev(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
     TV_HIP(hipSetDevice(ix->device));
     if (!d_mask_words) n_allowed = ix->n;
     return search_device(ix, d_queries, nq, k, d_mask_words, n_allowed, d_out_scores, d_out_indices, out_k_eff);
+}
+
+size_t tv_noalloc_scratch_bytes(void) { return kScratchBytes; }
+
+int tv_search_dev_noalloc(tv_index *ix, const float *d_queries, size_t nq, size_t k, const uint64_t *d_mask_words,
+                          size_t n_allowed, float *d_out_scores, int64_t *d_out_indices, size_t *out_k_eff) {
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    TV_HIP(hipSetDevice(ix->device));
+    if (!d_mask_words) n_allowed = ix->n;
+    const size_t k_eff = std::min(std::min(k, ix->n), n_allowed);
+    // What the search may carve, worst case: the sampled path's chunk, and the exact path a query
+    // falls back to when its candidates overflow.  Refused up front when that exceeds the array.
+    size_t need = 0;
+    if (k_eff != 0 && nq != 0) {
+        const size_t cq = std::min(nq, kChunkQueries);
+        need = robust_need(ix, cq, k_eff);
+        if (k_eff <= size_t(tv::kMaxSampledK) && !ix->force_robust) need = std::max(need, sampled_plan(ix, cq).need);
+    }
+    if (need > kScratchBytes) {
+        g_last_error = "tv_search_dev_noalloc: " + std::to_string(nq) + " queries, k=" + std::to_string(k) + " over " +
+                       std::to_string(ix->n) + " rows may need " + std::to_string(need) +
+                       " bytes of scratch; the fixed buffer holds " + std::to_string(kScratchBytes) +
+                       " (fewer queries per call; k <= 32 on a large index)";
+        return TV_ERR_BAD_ARGUMENT;
+    }
+    std::lock_guard<std::mutex> device_lock(g_scratch[ix->device].in_use);
+    void *own_ws = ix->ws;
+    const size_t own_bytes = ix->ws_bytes;
+    ix->ws = ix->scratch;
+    ix->ws_bytes = kScratchBytes;
+    ix->ws_fixed = true;
+    const int rc = search_device(ix, d_queries, nq, k, d_mask_words, n_allowed, d_out_scores, d_out_indices, out_k_eff);
+    ix->ws = own_ws;
+    ix->ws_bytes = own_bytes;
+    ix->ws_fixed = false;
+    return rc;
 }
 
 int tv_search(tv_index *ix, const float *queries, size_t nq, size_t k, const uint64_t *mask_words,

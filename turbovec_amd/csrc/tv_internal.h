@@ -167,6 +167,9 @@ struct tv_index {
     void *io = nullptr;            // staging for tv_search's host buffers (queries, mask, results); grows, never shrinks
     size_t io_bytes = 0;
     size_t ws_bytes = 0;
+    bool ws_fixed = false;         // ws is a lent buffer of fixed size (tv_search_dev_noalloc): never reallocated
+    void *scratch = nullptr;       // this device's copy of the library's static scratch array
+    uint32_t *h_flags = nullptr;   // pinned host memory: the overflow flags of one chunk of queries
     float last_scan_ms = 0.0f;
     int last_scan_launches = 0;
     int last_queries_per_launch = 0;   // queries one full-scan launch of the last search served
