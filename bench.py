@@ -58,6 +58,8 @@ def parse():
                          "instead of the all-queries-per-pass one")
     ap.add_argument("--cpu-sample", type=int, default=2_000_000, help="vectors in the CPU-baseline sample (0 = skip)")
     ap.add_argument("--cpu-threads", type=int, default=16)
+    ap.add_argument("--no-config3", action="store_true",
+                    help="skip the extra key for configuration 3 (10M x 1536 2-bit, k=100, batches 1 and 1024)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run the plain copy kernel over a 4 GiB buffer (counter calibration) and exit")
     return ap.parse_args()
@@ -99,6 +101,27 @@ def cpu_baseline(args):
     }
 
 
+def config3_extra(T, torch, build_index, run, args):
+    """Configuration 3 beside the headline: 10M x 1536 2-bit, k=100 (u8 LUT, u32 epilogue), batches 1
+    and 1024, each with the HBM roofline of its scan launch (algorithmic bytes = codes + row scales)."""
+    n, dim, bits, k = 10_000_000, 1536, 2, 100
+    ix = build_index(dim, bits, n)
+    alg = ((n + 31) // 32) * (dim // 4) * 32 + 4 * n
+    res = {"workload": f"TurboQuantIndex {n}x{dim} {bits}-bit, k={k}, no filter", "dtype": "u8",
+           "algorithmic_bytes_per_launch": alg}
+    for nq, steps in ((1024, max(3, args.steps // 2)), (1, max(args.steps, 15))):
+        dt, scan_ms, launches, q_full = run(nq, steps, 1, ix=ix, k=k, dim=dim)
+        launch_s = scan_ms * 1e-3 / max(launches, 1)
+        res[f"batch{nq}"] = {"queries_per_s": nq * steps / dt, "ms_per_step": dt / steps * 1e3,
+                             "queries_per_launch": q_full, "scan_launch_ms": launch_s * 1e3,
+                             "roofline": {"bound": "hbm", "achieved": alg / launch_s / 1e9, "peak": 8000.0,
+                                          "unit": "GB/s", "frac": alg / launch_s / 1e9 / 8000.0,
+                                          "traffic": None, "kernel": "k_scan_lut"}}
+    res["overflow_redos"] = ix.overflow_redos()
+    ix.close()
+    return res
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -123,27 +146,32 @@ def main():
     n_blocks = (n + 31) // 32
     gen = torch.Generator(device=dev)
     gen.manual_seed(0)
-    ix = T.NativeIndex(dim, bits)
+
+    def build_index(dim, bits, n):
+        # 100k-row chunks of unit Gaussian rows, generated and encoded on the device (tv_index_add_dev)
+        ix = T.NativeIndex(dim, bits)
+        for c0 in range(0, n, 100_000):
+            v = torch.randn(min(100_000, n - c0), dim, device=dev, generator=gen)
+            v = (v / v.norm(dim=1, keepdim=True)).contiguous()
+            torch.cuda.synchronize()
+            ix.add_dev(v.data_ptr(), v.shape[0])
+        del v
+        torch.cuda.empty_cache()
+        return ix
+
+    ix = build_index(dim, bits, n)
     if args.tile_groups:
         ix.set_path(4)
     if args.score_mode == "lut":
         ix.set_score_mode(T.SCORE_L_CLASSIC)
     mode_p = bits == 4 and args.score_mode == "auto"
-    # 100k-row chunks of unit Gaussian rows, generated and encoded on the device (tv_index_add_dev)
-    for c0 in range(0, n, 100_000):
-        v = torch.randn(min(100_000, n - c0), dim, device=dev, generator=gen)
-        v = (v / v.norm(dim=1, keepdim=True)).contiguous()
-        torch.cuda.synchronize()
-        ix.add_dev(v.data_ptr(), v.shape[0])
-    del v
-    torch.cuda.empty_cache()
 
-    def make_queries(nq):
+    def make_queries(nq, dim=dim):
         q = torch.randn(nq, dim, device=dev, generator=gen)
         return q / q.norm(dim=1, keepdim=True)
 
-    def run(nq, steps, warmup):
-        q = make_queries(nq)
+    def run(nq, steps, warmup, ix=ix, k=k, dim=dim):
+        q = make_queries(nq, dim)
         # the library works on its own stream: buffers handed to a _dev entry point must be complete
         torch.cuda.synchronize()
         out_s = torch.empty(nq, k, device=dev)
@@ -203,7 +231,8 @@ def main():
     int8_ops = 2.0 * q_per_launch * n * dim        # multiply-adds x2 of one launch, permute-dot mode
 
     out = {
-        "metric": "queries/sec, 10Mx1536 4-bit, k=10 (batch 1024; batch 1 beside it)",
+        "metric": "queries/sec, 10Mx1536 4-bit, k=10, batch 1024, inputs and outputs resident in HBM (tv_search_dev); "
+                  "host_buffers = the boundary call tv_search with PCIe copies, median of 5; batch1 beside it",
         "value": value,
         "unit": "queries/s",
         "n_gpus": 1,
@@ -252,6 +281,14 @@ def main():
                                               "algorithmic_bytes_per_launch", "achievable_read_GBps")}
         else:
             out["mfma"] = mfma
+    # queries of the timed steps that left the sampled path for the exact one (candidate overflow);
+    # Gaussian rows never do, and a non-zero count would mean the timed steps include that path's cost
+    out["overflow_redos"] = ix.overflow_redos()
+    if not args.no_config3 and (n, dim, bits) == (10_000_000, 1536, 4) and not args.tile_groups:
+        ix.close()
+        del ix
+        torch.cuda.empty_cache()
+        out["config3"] = config3_extra(T, torch, build_index, run, args)
     if args.cpu_sample > 0:
         out["cpu_baseline"] = cpu_baseline(args)
     print(json.dumps(out))
