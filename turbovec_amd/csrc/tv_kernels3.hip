@@ -56,6 +56,27 @@ __device__ __forceinline__ void lds_wait(v4i &r) {
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(r) : "n"(N));
 }
 
+// The int8 MFMA as hand-written instructions, for the forms of the kernel whose A operands do not
+// all fit the vector registers: an operand the compiler keeps in an accumulation register is copied
+// to a vector register before every use (four moves per MFMA, on the one wave of the SIMD that also
+// has to issue the MFMAs), while the instruction itself can read it where it is.  ACC_REG picks
+// the register file of the A operand; the accumulator stays in vector registers.  The compiler does
+// not know these are matrix instructions: the wait before their result is read is written out
+// (mfma_settle), and a tile's first MFMA takes the constant zero as its addend.
+template <bool ACC_REG>
+__device__ __forceinline__ void mfma_i8_first(v16i &acc, const v4i &a, const v4i &b) {
+    if constexpr (ACC_REG) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0" : "=&v"(acc) : "a"(a), "v"(b));
+    else asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
+}
+template <bool ACC_REG>
+__device__ __forceinline__ void mfma_i8_add(v16i &acc, const v4i &a, const v4i &b) {
+    if constexpr (ACC_REG) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(acc) : "a"(a), "v"(b));
+    else asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+}
+// An 8-pass MFMA's result may be read by the vector ALU 11 wait states after the instruction at
+// the earliest; 20 are spent.
+__device__ __forceinline__ void mfma_settle(v16i &acc) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(acc)); }
+
 // Per query, in LDS.  A score is fmaf(float(acc), qs, qb) * row_scale and passes when it reaches
 // tau.  With tau, qs > 0 and row scales >= 0 that needs acc >= (tau / max_row_scale - qb) / qs, up
 // to rounding: ta / max_row_scale - tb is that bound in accumulator units with the roundings of
@@ -72,13 +93,14 @@ struct WideQuery {
 
 // WAVES = 8 (two per SIMD, 256 VGPRs each) holds rows of up to 24 chunks; WAVES = 4 (one per SIMD)
 // gives a wave the whole 512-register file -- the compiler keeps what does not fit the VGPRs in
-// AGPRs, which the MFMA reads as A operands directly -- for rows of up to 48 chunks.  A tile's
-// weights go through the ring in SPT slices of NCH / SPT chunks.  Short rows leave registers
+// AGPRs -- for rows of up to 48 chunks.  A tile's weights go through the ring in SPT slices of
+// NCH / SPT chunks, handed over one by one (HO = 1) or HO at a time.  Short rows leave registers
 // for BLK blocks per wave: every B operand read from LDS then feeds BLK MFMAs, and a tile's
 // barriers and epilogue are shared by BLK times the work.
-template <int NCH, int NB, int WAVES, int SPT, int BLK>
+template <int NCH, int NB, int WAVES, int SPT, int BLK, int HO>
 __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide(ScanArgs a) {
     static_assert(NCH % SPT == 0, "a slice is a whole number of chunks");
+    static_assert(HO == 1 || (SPT % HO == 0 && kWideRing >= 2 * HO + 1), "slices handed over together must fit the ring twice");
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr int kWideThreads = WAVES * 64, kWideWaves = WAVES;
     constexpr int kSC = NCH / SPT;                          // chunks per slice
@@ -87,6 +109,11 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     constexpr int kPieces = kM / kWideWaves;                // direct-to-LDS loads per wave and slice ...
     constexpr int kExtra = kM % kWideWaves;                 // ... plus one more in the first kExtra waves
     constexpr int kAhead = kWideRing - 1;
+    // Four-wave forms (one wave per SIMD, up to 48 chunks = 384 operand registers): chunks from
+    // kVecChunks on live in accumulation registers and the MFMAs are written by hand.
+    constexpr bool kHandMfma = WAVES == 4 && BLK == 1;
+    constexpr int kVecChunks = 22;
+    static_assert(!kHandMfma || (NCH - kVecChunks) * 8 <= 256, "operands beyond the vector registers must fit the accumulation registers");
     const int nq = a.nq_tile;
     const int nt = (nq + kQTile - 1) / kQTile;
     const int nq_pad = nt * kQTile;
@@ -168,9 +195,27 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
         __syncthreads();
         request_next();
     };
-    // slices 0..3 requested, slice 0 whole: the state the first hand-over expects
-    for (int i = 0; i < kAhead - 1; ++i) request_next();
-    hand_over(IntC<kAhead - 2>{});
+    // HO > 1: one hand-over per HO slices, in the middle of the last of them.  By then every wave
+    // is past slices g - HO .. g - 1 (g = the slice in progress); each wave's pieces of the HO
+    // slices after g, requested at the hand-over before, must have landed (nothing younger is in
+    // flight: the wait is for everything); after the barrier those are whole and the HO slices
+    // behind g are free: the next HO slices are requested into their slots.
+    auto hand_over_group = [&]() {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < HO; ++i) request_next();
+    };
+    if constexpr (HO == 1) {
+        // slices 0..3 requested, slice 0 whole: the state the first hand-over expects
+        for (int i = 0; i < kAhead - 1; ++i) request_next();
+        hand_over(IntC<kAhead - 2>{});
+    } else {
+        // slices 0 .. 2 HO - 1 requested and whole: the state the first group hand-over expects
+        for (int i = 0; i < 2 * HO; ++i) request_next();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
     int use_slot = 0;                                       // ring slot of the slice consumed next
 
     v4i alo[BLK][NCH], ahi[BLK][NCH];
@@ -197,14 +242,23 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
         const uint32_t naddr = lds_b + uint32_t(use_slot) * kSlice + lane16;
         static_for<kM>([&](auto mm) {
             constexpr int m = decltype(mm)::value;
-            if constexpr (m == kM / 2) hand_over(IntC<kAhead - 2>{});
+            if constexpr (m == kM / 2) {
+                if constexpr (HO == 1) hand_over(IntC<kAhead - 2>{});
+                else if constexpr (decltype(part)::value % HO == HO - 1) hand_over_group();
+            }
             lds_wait<NB - 1>(w[m % NB]);
             static_for<BLK>([&](auto kk) {
                 constexpr int k = decltype(kk)::value;
-                if constexpr ((m & 1) == 0)
-                    acc[k] = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo[k][c0 + m / 2], w[m % NB], acc[k], 0, 0, 0);
-                else
-                    acc[k] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi[k][c0 + m / 2], w[m % NB], acc[k], 0, 0, 0);
+                constexpr int c = c0 + m / 2;
+                if constexpr (kHandMfma) {
+                    const v4i &A = (m & 1) == 0 ? alo[k][c] : ahi[k][c];
+                    if constexpr (decltype(part)::value == 0 && m == 0) mfma_i8_first<(c >= kVecChunks)>(acc[k], A, w[m % NB]);
+                    else mfma_i8_add<(c >= kVecChunks)>(acc[k], A, w[m % NB]);
+                } else if constexpr ((m & 1) == 0) {
+                    acc[k] = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo[k][c], w[m % NB], acc[k], 0, 0, 0);
+                } else {
+                    acc[k] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi[k][c], w[m % NB], acc[k], 0, 0, 0);
+                }
             });
             if constexpr (m + NB < kM) lds_read16_async<(m + NB) * 1024>(w[m % NB], baddr);
             else lds_read16_async<(m + NB - kM) * 1024>(w[m % NB], naddr);
@@ -232,18 +286,26 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
                 // chunk) fit the registers the operands alone need at the end
                 const uint8_t *p = a.codes + size_t(b) * NCH * 1024;
                 u32x4 raw[NCH];
-                static_for<NCH>([&](auto cc) {
-                    constexpr int c = decltype(cc)::value;
+                // with hand-written MFMAs the chunks bound for the accumulation registers come
+                // first: their raw codes leave the vector registers before the others' operands grow
+                constexpr int kFirst = kHandMfma && NCH > kVecChunks ? kVecChunks : 0;
+                static_for<NCH>([&](auto ii) {
+                    constexpr int c = (decltype(ii)::value + kFirst) % NCH;
                     load16_async_s(raw[c], p + size_t(c) * 1024, lane16);
                 });
-                static_for<NCH>([&](auto cc) {
-                    constexpr int c = decltype(cc)::value;
-                    wait_vm<NCH - 1 - c>(raw[c]);
+                static_for<NCH>([&](auto ii) {
+                    constexpr int c = (decltype(ii)::value + kFirst) % NCH;
+                    wait_vm<NCH - 1 - decltype(ii)::value>(raw[c]);
                     const uint32_t x[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
 #pragma unroll
                     for (int d = 0; d < 4; ++d) {
                         alo[k][c][d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
                         ahi[k][c][d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
+                    }
+                    if constexpr (kHandMfma && c >= kVecChunks) {
+                        // into its accumulation registers now, not at the first MFMA that reads it
+                        asm volatile("" : "+a"(alo[k][c]));
+                        asm volatile("" : "+a"(ahi[k][c]));
                     }
                 });
                 const uint32_t slot = b * 32u + uint32_t(lane & 31);
@@ -298,7 +360,8 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
         for (int t = 0; t < nt; ++t) {
             const int q = t * kQTile + qn;
             if (has) {
-                static_for<BLK>([&](auto kk) { acc[decltype(kk)::value] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}; });
+                if constexpr (!kHandMfma)
+                    static_for<BLK>([&](auto kk) { acc[decltype(kk)::value] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}; });
                 slice_mfmas(IntC<0>{});
                 // the tile's accumulator bounds, fetched and converted under the MFMAs
                 const float2 tq = *reinterpret_cast<const float2 *>(&sq[q].ta);
@@ -312,6 +375,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
                 static_for<SPT - 1>([&](auto pp) { slice_mfmas(IntC<decltype(pp)::value + 1>{}); });
                 static_for<BLK>([&](auto kk) {
                     constexpr int k = decltype(kk)::value;
+                    if constexpr (kHandMfma) mfma_settle(acc[k]);
                     const v16i &c = acc[k];
                     int m0 = max(max(c[0], c[1]), c[2]), m1 = max(max(c[3], c[4]), c[5]);
                     int m2 = max(max(c[6], c[7]), c[8]), m3 = max(max(c[9], c[10]), c[11]);
@@ -321,8 +385,13 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
                 });
             } else {
                 use_slot = (use_slot + SPT) % kWideRing;
+                if constexpr (HO == 1) {
 #pragma unroll
-                for (int i = 0; i < SPT; ++i) hand_over(IntC<kAhead - 2>{});
+                    for (int i = 0; i < SPT; ++i) hand_over(IntC<kAhead - 2>{});
+                } else {
+#pragma unroll
+                    for (int i = 0; i < SPT / HO; ++i) hand_over_group();
+                }
             }
         }
         if (has) close_stream();
@@ -412,15 +481,15 @@ int wide_grid_blocks(int device) {
     return cus;      // one 8-wave workgroup per CU: its LDS holds the slice ring
 }
 
-template <int NCH, int NB, int WAVES = 8, int SPT = 2, int BLK = 1>
+template <int NCH, int NB, int WAVES = 8, int SPT = 2, int BLK = 1, int HO = 1>
 static hipError_t launch_wide_n(const ScanArgs &a, int grid, hipStream_t s) {
     const size_t lds = wide_lds_bytes(2 * (NCH / SPT) * 1024, a.nq_tile, BLK);
     if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK, HO>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK>), dim3(grid), dim3(WAVES * 64), lds, s, a);
+    hipLaunchKernelGGL((k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK, HO>), dim3(grid), dim3(WAVES * 64), lds, s, a);
     return hipGetLastError();
 }
 
@@ -428,19 +497,21 @@ static hipError_t launch_wide_n(const ScanArgs &a, int grid, hipStream_t s) {
 // ceil(nq/32) weight tiles back to back, a.qscale / a.qbias / a.gtau indexed by query.
 hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s) {
     switch (a.nch) {
-        // <chunks, B-operand registers, waves, slices per tile, blocks per wave>
+        // <chunks, B-operand registers, waves, slices per tile, blocks per wave, slices per hand-over>
+        // One hand-over per tile (two slices) measured 2.5 to 5 % faster than one per slice in the
+        // eight-wave forms with two slices per tile, and 2 % slower in the four-wave forms.
         case 2: return launch_wide_n<2, 2, 8, 1, 6>(a, grid, s);
         case 4: return launch_wide_n<4, 2, 8, 1, 4>(a, grid, s);
         case 6: return launch_wide_n<6, 2, 8, 1, 3>(a, grid, s);
         case 8: return launch_wide_n<8, 4, 8, 1, 2>(a, grid, s);
-        case 10: return launch_wide_n<10, 2, 8, 2, 2>(a, grid, s);
-        case 12: return launch_wide_n<12, 2, 8, 2, 2>(a, grid, s);
-        case 14: return launch_wide_n<14, 2, 8, 2, 1>(a, grid, s);
-        case 16: return launch_wide_n<16, 4, 8, 2, 1>(a, grid, s);
-        case 18: return launch_wide_n<18, 2, 8, 2, 1>(a, grid, s);
-        case 20: return launch_wide_n<20, 4, 8, 2, 1>(a, grid, s);
-        case 22: return launch_wide_n<22, 2, 8, 2, 1>(a, grid, s);
-        case 24: return launch_wide_n<24, 2, 8, 2, 1>(a, grid, s);
+        case 10: return launch_wide_n<10, 2, 8, 2, 2, 2>(a, grid, s);
+        case 12: return launch_wide_n<12, 2, 8, 2, 2, 2>(a, grid, s);
+        case 14: return launch_wide_n<14, 2, 8, 2, 1, 2>(a, grid, s);
+        case 16: return launch_wide_n<16, 4, 8, 2, 1, 2>(a, grid, s);
+        case 18: return launch_wide_n<18, 2, 8, 2, 1, 2>(a, grid, s);
+        case 20: return launch_wide_n<20, 4, 8, 2, 1, 2>(a, grid, s);
+        case 22: return launch_wide_n<22, 2, 8, 2, 1, 2>(a, grid, s);
+        case 24: return launch_wide_n<24, 2, 8, 2, 1, 2>(a, grid, s);
         case 28: return launch_wide_n<28, 2, 4, 4, 1>(a, grid, s);
         case 32: return launch_wide_n<32, 4, 4, 4, 1>(a, grid, s);
         case 36: return launch_wide_n<36, 2, 4, 4, 1>(a, grid, s);
