@@ -358,6 +358,149 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
     }
 }
 
+// ===========================================================================
+// Single-query scan over byte tables, score modes L, append mode.
+//
+// With one query the two nibble tables of a byte-group (16 entries each) are first folded
+// into one 256-entry table per code byte in LDS -- entry b = lut[hi nibble of b] +
+// lut[16 + lo nibble of b], at most 254, so still a byte -- and the scan then makes ONE LDS
+// read per code byte instead of two, addressed by the raw code byte (no nibble split).  The
+// integer sums are those of the two-read walk (turbovec/src/search.rs:3113-3128), term for
+// term, so the epilogues reproduce the reference's floats as before.  A byte table takes 256
+// bytes per byte-group (96 KiB at 1536 dimensions and 2 bits); rows too long for that get byte
+// tables for their first n_bt chunks and keep the two nibble reads for the rest (19 of 24
+// chunks at 1536 dimensions and 4 bits).
+// ===========================================================================
+constexpr int kLutBtThreads = 1024;
+
+template <int U>
+__global__ __launch_bounds__(kLutBtThreads) void k_scan_lut_bt(ScanArgs a, int n_bt) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int nch = a.nch;
+    uint8_t *bt = smem;                                                   // [n_bt * 32][256]
+    uint8_t *nt = smem + size_t(n_bt) * 8192;                             // [(nch - n_bt) * 32][32]: the nibble tables as built
+    uint32_t *scnt = reinterpret_cast<uint32_t *>(nt + size_t(nch - n_bt) * 1024);
+    const int tid = threadIdx.x;
+    // fold: four entries (one dword) per step
+    for (int w = tid; w < n_bt * 32 * 64; w += kLutBtThreads) {
+        const int g = w >> 6, b0 = (w & 63) * 4;
+        const uint8_t *row = a.tables + size_t(g) * 32;
+        const uint32_t hi = row[b0 >> 4];
+        uint32_t v = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v |= (hi + uint32_t(row[16 + ((b0 + e) & 15)])) << (8 * e);
+        reinterpret_cast<uint32_t *>(bt)[w] = v;
+    }
+    for (int w = tid; w < (nch - n_bt) * 256; w += kLutBtThreads)
+        reinterpret_cast<uint32_t *>(nt)[w] = reinterpret_cast<const uint32_t *>(a.tables + size_t(n_bt) * 1024)[w];
+    if (tid == 0) *scnt = 0u;
+    __syncthreads();
+    typedef const __attribute__((address_space(3))) uint8_t lds_byte_t;
+    const uint32_t lds_bt = uint32_t(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)smem));
+    const uint32_t lds_nt = lds_bt + uint32_t(n_bt) * 8192;
+
+    const int lane = tid & 63, wave = tid >> 6;
+    const int vi = lane & 31, h = lane >> 5;
+    const float qs = a.qscale[0], qb = a.qbias[0];
+    const float tau = order_unkey(a.gtau[0]);
+    const uint32_t step = a.b_step;
+    const uint32_t nj = (a.n_blocks + step - 1) / step;
+    const uint32_t total_waves = gridDim.x * (kLutBtThreads / 64);
+    const uint4 *codes = reinterpret_cast<const uint4 *>(a.codes) + lane;
+
+    auto live_from = [&](uint32_t j) -> uint32_t {
+        if (a.mask == nullptr) return j;
+        while (j < nj) {
+            const uint32_t b = j * step;
+            if (uint32_t(a.mask[b >> 1] >> ((b & 1) * 32)) != 0u) break;
+            j += total_waves;
+        }
+        return j;
+    };
+
+    uint32_t j = live_from(wave * gridDim.x + blockIdx.x);   // consecutive blocks go to different workgroups
+    uint4 buf[U];
+    if (j < nj) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) buf[u] = load_stream16(&codes[(size_t(j) * step * nch + u) * 64]);
+    }
+    while (j < nj) {
+        const uint32_t nj_live = live_from(j + total_waves);
+        const uint32_t b = j * step;
+        uint32_t total = 0, acc = 0;
+        float fa = qb;
+        for (int c0 = 0; c0 < nch; c0 += U) {
+            uint4 cur[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) cur[u] = buf[u];
+            if (c0 + U < nch) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) buf[u] = load_stream16(&codes[(size_t(b) * nch + c0 + U + u) * 64]);
+            } else if (nj_live < nj) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) buf[u] = load_stream16(&codes[(size_t(nj_live) * step * nch + u) * 64]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u;
+                const uint32_t x[4] = {cur[u].x, cur[u].y, cur[u].z, cur[u].w};
+                if (c < n_bt) {
+                    const uint32_t row_off = lds_bt + uint32_t(c * 32 + 16 * h) * 256;
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        static_for4([&](auto ec) {
+                            constexpr int e = decltype(ec)::value;
+                            acc += uint32_t(*reinterpret_cast<lds_byte_t *>(add_byte<e>(row_off, x[d]) + (d * 4 + e) * 256));
+                        });
+                    }
+                } else {
+                    const uint32_t row_off = lds_nt + uint32_t((c - n_bt) * 32 + 16 * h) * 32;
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        const uint32_t plo = x[d] & 0x0f0f0f0fu, phi = (x[d] >> 4) & 0x0f0f0f0fu;
+                        static_for4([&](auto ec) {
+                            constexpr int e = decltype(ec)::value;
+                            acc += uint32_t(*reinterpret_cast<lds_byte_t *>(add_byte<e>(row_off, phi) + (d * 4 + e) * 32));
+                            acc += uint32_t(*reinterpret_cast<lds_byte_t *>(add_byte<e>(row_off, plo) + (d * 4 + e) * 32 + 16));
+                        });
+                    }
+                }
+                if ((c & 7) == 7 || c == nch - 1) {  // end of a 256-group batch (search.rs:529-531)
+                    const uint32_t part = acc + uint32_t(__shfl_xor(int(acc), 32));
+                    acc = 0;
+                    total += part;
+                    fa = fmaf(qs, float(part), fa);   // search.rs:577-580
+                }
+            }
+        }
+        const uint32_t slot0 = b * 32u;
+        uint32_t mw = 0xffffffffu;
+        if (a.mask != nullptr) mw = uint32_t(a.mask[b >> 1] >> ((b & 1) * 32));
+        const uint32_t slot = slot0 + uint32_t(vi);
+        if (h == 0 && slot < a.n && ((mw >> vi) & 1u)) {
+            const float vs = a.scales[slot];
+            // classic: fa * vec_scale; u32: ((f32(acc) * scale) + bias) * vec_scale (search.rs:1174-1177)
+            const float sc = a.classic ? fa * vs : ((float(int(total)) * qs) + qb) * vs;
+            if (sc >= tau) {
+                const uint32_t pos = atomicAdd(scnt, 1u);
+                if (pos < kSegCap) a.cand[size_t(blockIdx.x) * kSegCap + pos] = sort_key(sc, slot);
+            }
+        }
+        j = nj_live;
+    }
+    __syncthreads();
+    if (tid == 0) a.cand_cnt[blockIdx.x] = *scnt;
+}
+
+// Chunks of a row that get byte tables when `budget` bytes of LDS are available, and the bytes used.
+static int lut_bt_chunks(int nch, size_t budget) {
+    const size_t fixed = size_t(nch) * 1024 + 64;
+    if (budget <= fixed) return 0;
+    const size_t n = (budget - fixed) / (8192 - 1024);
+    return int(n < size_t(nch) ? n : size_t(nch));
+}
+static size_t lut_bt_lds_bytes(int nch, int n_bt) { return size_t(n_bt) * 8192 + size_t(nch - n_bt) * 1024 + 64; }
+
 static constexpr size_t kLdsBudgetL = 160 * 1024;
 
 static size_t lut_lds_bytes(int nch, int k, int ql, bool no_lists, int threads) {
@@ -382,11 +525,14 @@ int lut_append_queries(int nch) {
     return 1;
 }
 
+static int lut_cus = 256;   // compute units of the device the last grid was sized for
+
 int lut_append_grid(int device, int nch) {
     hipDeviceProp_t prop;
     int cus = 256;
     if (hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0)
         cus = prop.multiProcessorCount;
+    lut_cus = cus;
     const size_t lds = lut_lds_bytes(nch, 0, lut_append_queries(nch), true, kLutAppendThreads);
     return cus * (lds * 2 <= kLdsBudgetL ? 2 : 1);   // at most 2048 threads per CU
 }
@@ -408,6 +554,25 @@ int lut_launch_ql(int nch, int k, int nq_tile) {
 // lut_tile_queries(nch, k) otherwise.
 hipError_t launch_scan_lut(const ScanArgs &a, int grid, int mode, hipStream_t s) {
     const bool append = mode == kModeAppend;
+    if (append && a.nq_tile == 1) {
+        // one query: byte tables for as many chunks as fit, one LDS read per code byte there
+        const int n_bt = lut_bt_chunks(a.nch, grid > lut_cus ? kLdsBudgetL / 2 : kLdsBudgetL);
+        if (n_bt * 2 >= a.nch) {
+            const size_t lds = lut_bt_lds_bytes(a.nch, n_bt);
+            hipError_t e = hipSuccess;
+#define TV_LAUNCH_BT(U)                                                                          \
+            do {                                                                                 \
+                e = allow_lds2(k_scan_lut_bt<U>, lds);                                           \
+                if (e != hipSuccess) return e;                                                   \
+                hipLaunchKernelGGL(k_scan_lut_bt<U>, dim3(grid), dim3(kLutBtThreads), lds, s, a, n_bt); \
+            } while (0)
+            if (a.nch % 4 == 0) TV_LAUNCH_BT(4);
+            else if (a.nch % 2 == 0) TV_LAUNCH_BT(2);
+            else TV_LAUNCH_BT(1);
+#undef TV_LAUNCH_BT
+            return hipGetLastError();
+        }
+    }
     const bool dump = mode != kModeLists;   // no list storage in LDS
     const int kk = a.k;                     // the tile width is chosen for the list pass of the same search
     const int threads = append ? kLutAppendThreads : kLutListThreads;
