@@ -67,6 +67,9 @@ def _load():
     lib.tvo_search.argtypes = [i32, f32p, sz, vp, vp, f32p, f32p, f32p, f32p, i32, i32, sz, sz, vp,
                                f32p, vp, vp, vp, f32p, i32]
     lib.tvo_search_fast.argtypes = [f32p, sz, vp, vp, f32p, f32p, i32, i32, sz, sz, vp, f32p, vp, vp, i32]
+    lib.tvo_have_vnni.restype = i32
+    lib.tvo_seq_to_vector_major.argtypes = [vp, sz, i32, i32, vp]
+    lib.tvo_search_vnni.argtypes = [f32p, sz, vp, vp, f32p, f32p, i32, sz, sz, vp, f32p, vp, vp, i32]
     lib.tvo_validate_queries.argtypes = [f32p, sz, i32, vp]
     lib.tvo_pack_mask.restype = sz
     lib.tvo_pack_mask.argtypes = [vp, sz, vp]
@@ -287,6 +290,42 @@ def search_fast(rot, seq, scales, queries, k, bits, dim, n, mask_words=None, n_t
                                _p(mask_words), _p(out_s), _p(out_i), C.addressof(k_eff), n_threads)
     if rc != 0:
         raise RuntimeError(f"tvo_search_fast failed rc={rc}")
+    return out_s, out_i
+
+
+def have_vnni():
+    return bool(lib().tvo_have_vnni())
+
+
+def seq_to_vector_major(seq, n, bits, dim):
+    """The layout the reference keeps at rest on VNNI hosts (pack.rs:1269-1271, :1347-1358)."""
+    seq = np.ascontiguousarray(seq, np.uint8)
+    out = np.zeros_like(seq)
+    if lib().tvo_seq_to_vector_major(_p(seq), n, bits, dim, _p(out)) != 0:
+        raise ValueError("vector-major needs a multiple of 4 byte-groups")
+    return out
+
+
+def search_vnni(rot, vm, scales, queries, k, dim, n, mask_words=None, n_threads=8):
+    """The reference's AVX-512 VNNI permute-dot kernel (4-bit) over vector-major codes."""
+    q = _f32(queries).reshape(-1, dim)
+    nq = q.shape[0]
+    _, cen = codebook(4, dim)
+    vm = np.ascontiguousarray(vm, np.uint8)
+    scales = _f32(scales)
+    n_allowed = n
+    if mask_words is not None:
+        mask_words = np.ascontiguousarray(mask_words, np.uint64)
+        n_allowed = int(np.unpackbits(mask_words.view(np.uint8)).sum())
+    kk = min(k, n, n_allowed)
+    assert kk <= 1024
+    out_s = np.zeros((nq, kk), np.float32)
+    out_i = np.zeros((nq, kk), np.int64)
+    k_eff = C.c_size_t(0)
+    rc = lib().tvo_search_vnni(_p(q), nq, rot.h, _p(vm), _p(cen), _p(scales), dim, n, k,
+                               _p(mask_words), _p(out_s), _p(out_i), C.addressof(k_eff), n_threads)
+    if rc != 0:
+        raise RuntimeError(f"tvo_search_vnni failed rc={rc}")
     return out_s, out_i
 
 

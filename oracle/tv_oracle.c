@@ -984,6 +984,240 @@ int tvo_search_fast(const float *queries, size_t nq, const tvo_rotation *rot,
 }
 
 /* ======================================================================= */
+/* The reference's production kernel for 4-bit on AVX-512 VNNI hosts:        */
+/* search_multi_query_permute_dot (search.rs:1392-1567) over the             */
+/* vector-major layout (pack.rs:1269-1271, :1347-1358), eight queries per    */
+/* pass over a block.  Same integers and floats as tvo_search mode P (tests  */
+/* compare them); this is what the CPU-baseline timing runs when the host    */
+/* has the instructions, so that the baseline runs the reference's           */
+/* algorithm at the reference's speed.                                       */
+/* ======================================================================= */
+
+/* pack.rs:1347-1358 vector_major_chunk over every unit of 4 byte-groups x 32 vectors:
+ * byte of (group 4*q4 + j, vector v) moves to q4*128 + (v/16)*64 + (v%16)*4 + j.
+ * dim*bits/8 must be a multiple of 4 (pack.rs:1260-1263).  Out of place. */
+int tvo_seq_to_vector_major(const uint8_t *seq, size_t n, int bits, int dim, uint8_t *vm) {
+    size_t G = tvo_n_byte_groups(bits, dim);
+    if (G % 4 != 0) return TVO_ERR_BAD_ARGUMENT;
+    size_t n_units = (n + TVO_BLOCK - 1) / TVO_BLOCK * (G / 4);
+    for (size_t u = 0; u < n_units; u++) {
+        const uint8_t *src = seq + u * 128;
+        uint8_t *dst = vm + u * 128;
+        for (int j = 0; j < 4; j++)
+            for (int v = 0; v < TVO_BLOCK; v++) dst[(v / 16) * 64 + (v % 16) * 4 + j] = src[j * TVO_BLOCK + v];
+    }
+    return TVO_OK;
+}
+
+#if defined(__x86_64__)
+#include <immintrin.h>
+
+int tvo_have_vnni(void) {
+    __builtin_cpu_init();
+    return __builtin_cpu_supports("avx512f") && __builtin_cpu_supports("avx512bw") && __builtin_cpu_supports("avx512vnni");
+}
+
+#define TVO_NQ 8
+
+/* One block range, up to eight queries: search.rs:1417-1545.  w8: the queries' weights in the
+ * reference's quad layout ([q4*8 + j] = low-nibble weight of group 4*q4 + j, [q4*8 + 4 + j] = high). */
+__attribute__((target("avx2,fma,avx512f,avx512bw,avx512vnni"), always_inline))
+static inline void scan_range_vnni_n(const uint8_t *vm, size_t G, size_t b0, size_t b1, size_t n,
+                                     const int8_t *const *w8, const int32_t *zero, const float *qscale,
+                                     const float *qbias, const int nqm, const int8_t *levels16,
+                                     const float *vec_scales, const uint64_t *mask, heap_t *heaps, size_t k) {
+    const __m512i m0f = _mm512_set1_epi8(0x0F);
+    const size_t quads = G / 4, block_bytes = G * TVO_BLOCK;
+    /* +128 puts the signed levels into vpdpbusd's unsigned operand; `zero` cancels it (search.rs:1426-1429) */
+    const __m512i levels = _mm512_xor_si512(_mm512_broadcast_i32x4(_mm_loadu_si128((const __m128i *)levels16)),
+                                            _mm512_set1_epi8((char)0x80));
+    for (size_t b = b0; b < b1; b++) {
+        const size_t base_vec = b * TVO_BLOCK;
+        uint32_t mw = 0xFFFFFFFFu;
+        if (mask) { mw = (uint32_t)(mask[base_vec >> 6] >> (base_vec & 63)); if (!mw) continue; }   /* search.rs:3015-3029 */
+        const uint8_t *blk = vm + b * block_bytes;
+        __m512i acc[TVO_NQ][2];
+        for (int qi = 0; qi < nqm; qi++) { acc[qi][0] = _mm512_set1_epi32(zero[qi]); acc[qi][1] = acc[qi][0]; }
+        for (size_t q4 = 0; q4 < quads; q4++) {
+            for (int h = 0; h < 2; h++) {
+                const uint8_t *p = blk + q4 * 128 + (size_t)h * 64;
+                _mm_prefetch((const char *)(p + 32 * 128), _MM_HINT_T0);
+                const __m512i c = _mm512_loadu_si512((const void *)p);
+                const __m512i vlo = _mm512_shuffle_epi8(levels, _mm512_and_si512(c, m0f));
+                const __m512i vhi = _mm512_shuffle_epi8(levels, _mm512_and_si512(_mm512_srli_epi16(c, 4), m0f));
+                for (int qi = 0; qi < nqm; qi++) {
+                    int32_t wl, wh;
+                    memcpy(&wl, w8[qi] + q4 * 8, 4);
+                    memcpy(&wh, w8[qi] + q4 * 8 + 4, 4);
+                    acc[qi][h] = _mm512_dpbusd_epi32(acc[qi][h], vlo, _mm512_set1_epi32(wl));
+                    acc[qi][h] = _mm512_dpbusd_epi32(acc[qi][h], vhi, _mm512_set1_epi32(wh));
+                }
+            }
+        }
+        const size_t lanes = n - base_vec < TVO_BLOCK ? n - base_vec : TVO_BLOCK;
+        const int full = lanes == TVO_BLOCK;
+        float vsb[TVO_BLOCK];
+        for (size_t l = 0; l < TVO_BLOCK; l++) vsb[l] = l < lanes ? vec_scales[base_vec + l] : 0.0f;
+        for (int qi = 0; qi < nqm; qi++) {
+            /* search.rs:1519-1524: fma(f32(acc), scale, bias), then the row scale (:1793-1794) */
+            const __m512 vs = _mm512_set1_ps(qscale[qi]), vb = _mm512_set1_ps(qbias[qi]);
+            const __m512 s0 = _mm512_mul_ps(_mm512_fmadd_ps(_mm512_cvtepi32_ps(acc[qi][0]), vs, vb), _mm512_loadu_ps(vsb));
+            const __m512 s1 = _mm512_mul_ps(_mm512_fmadd_ps(_mm512_cvtepi32_ps(acc[qi][1]), vs, vb), _mm512_loadu_ps(vsb + 16));
+            heap_t *hp = &heaps[qi];
+            if (hp->sz >= k && full) {   /* search.rs:1792-1800: nothing in the block beats the heap's minimum */
+                const __m512 thr = _mm512_set1_ps(hp->mn);
+                if ((_mm512_cmp_ps_mask(s0, thr, _CMP_GT_OQ) | _mm512_cmp_ps_mask(s1, thr, _CMP_GT_OQ)) == 0) continue;
+            }
+            float out[TVO_BLOCK];
+            _mm512_storeu_ps(out, s0);
+            _mm512_storeu_ps(out + 16, s1);
+            for (size_t l = 0; l < lanes; l++) {
+                if (!((mw >> l) & 1)) continue;
+                heap_push(hp, k, out[l], base_vec + l);
+            }
+        }
+    }
+}
+
+/* The query count is a compile-time constant in each instance (the reference's const generic NQ),
+ * so the accumulators of all eight queries live in registers. */
+__attribute__((target("avx2,fma,avx512f,avx512bw,avx512vnni")))
+static void scan_range_vnni(const uint8_t *vm, size_t G, size_t b0, size_t b1, size_t n,
+                            const int8_t *const *w8, const int32_t *zero, const float *qscale,
+                            const float *qbias, int nqm, const int8_t *levels16,
+                            const float *vec_scales, const uint64_t *mask, heap_t *heaps, size_t k) {
+#define TVO_CASE(N) case N: scan_range_vnni_n(vm, G, b0, b1, n, w8, zero, qscale, qbias, N, levels16, vec_scales, mask, heaps, k); break
+    switch (nqm) {
+        TVO_CASE(1); TVO_CASE(2); TVO_CASE(3); TVO_CASE(4); TVO_CASE(5); TVO_CASE(6); TVO_CASE(7); TVO_CASE(8);
+        default: break;
+    }
+#undef TVO_CASE
+}
+#else
+int tvo_have_vnni(void) { return 0; }
+#endif
+
+/* search::search for 4-bit indexes held in the vector-major layout: block ranges over threads,
+ * inside a range eight queries per pass (search.rs:3996-4050), per-range heaps merged by
+ * (score desc, slot asc) (search.rs:4279-4298).  Uncalibrated indexes, k <= 1024.  Returns
+ * TVO_ERR_BAD_ARGUMENT when the host lacks AVX-512 VNNI. */
+int tvo_search_vnni(const float *queries, size_t nq, const tvo_rotation *rot,
+                    const uint8_t *vm_codes, const float *centroids, const float *vec_scales,
+                    int dim, size_t n, size_t k, const uint64_t *mask,
+                    float *out_scores, int64_t *out_indices, size_t *out_k_eff, int n_threads) {
+#if defined(__x86_64__)
+    if (!tvo_have_vnni()) return TVO_ERR_BAD_ARGUMENT;
+    const size_t G = (size_t)dim / 2;
+    if (G % 4 != 0) return TVO_ERR_BAD_ARGUMENT;
+    const size_t n_blocks = (n + TVO_BLOCK - 1) / TVO_BLOCK;
+    size_t n_allowed = n;
+    if (mask) {
+        n_allowed = 0;
+        for (size_t w = 0; w < (n + 63) / 64; w++) n_allowed += (size_t)__builtin_popcountll(mask[w]);
+    }
+    if (k > n_allowed) k = n_allowed;
+    if (k > n) k = n;
+    *out_k_eff = k;
+    if (k == 0 || nq == 0) return TVO_OK;
+    if (n_threads < 1) n_threads = 1;
+    int8_t *W = (int8_t *)malloc(nq * (size_t)dim);
+    int32_t *zero = (int32_t *)malloc(sizeof(int32_t) * nq);
+    float *qscale = (float *)malloc(sizeof(float) * nq), *qbias = (float *)calloc(nq, sizeof(float));
+    int8_t levels[16];
+#pragma omp parallel for schedule(static) num_threads(n_threads)
+    for (long long qi = 0; qi < (long long)nq; qi++) {
+        float *q_rot = (float *)malloc(sizeof(float) * (size_t)dim);
+        memcpy(q_rot, queries + (size_t)qi * dim, sizeof(float) * (size_t)dim);
+        tvo_rotation_apply(rot, q_rot);
+        int8_t lv[16];
+        tvo_build_permute_dot(q_rot, centroids, dim, lv, W + (size_t)qi * dim, &zero[qi], &qscale[qi]);
+        free(q_rot);
+    }
+    {
+        float cmax = 0.0f;
+        for (int i = 0; i < 16; i++) { float v = fabsf(centroids[i]); if (v > cmax) cmax = v; }
+        float cs = cmax > 0.0f ? cmax / 127.0f : 1.0f;
+        for (int i = 0; i < 16; i++) levels[i] = (int8_t)clampf(roundf(centroids[i] / cs), -127.0f, 127.0f);
+    }
+    /* Tiles = query groups of eight x block ranges, as the reference's batch dispatch cuts them
+     * (search.rs:125-144 n_block_ranges with TILES_PER_THREAD = 32 :178 and MIN_TILE_BLOCKS_X86 =
+     * 3072 :226, :265-278 range_cap_for_k, :284-295 smooth_tile_count; a mask keeps one range,
+     * :111-113), drawn block-range-major by the pool (search.rs:4031-4046). */
+    const size_t n_groups = (nq + TVO_NQ - 1) / TVO_NQ;
+    size_t n_ranges = 1;
+    if (n_threads > 1 && !mask) {
+        n_ranges = ((size_t)n_threads * 32 + n_groups - 1) / n_groups;
+        const size_t by_blocks = (n_blocks + 3071) / 3072;
+        size_t by_k = (n + 512 * k - 1) / (512 * k);
+        if (by_k < 1) by_k = 1;
+        if (n_ranges > by_blocks) n_ranges = by_blocks;
+        if (n_ranges > by_k) n_ranges = by_k;
+        if (n_ranges < 1) n_ranges = 1;
+        const size_t tiles = n_groups * n_ranges;
+        if (tiles > (size_t)n_threads && tiles < 2 * (size_t)n_threads) {
+            n_ranges = (size_t)n_threads / n_groups;
+            if (n_ranges < 1) n_ranges = 1;
+        }
+    }
+    size_t stride = (n_blocks + n_ranges - 1) / n_ranges;
+    if (stride < 1) stride = 1;
+    stride += stride & 1;                   /* ranges start on mask-word boundaries (search.rs:3038) */
+    n_ranges = (n_blocks + stride - 1) / stride;
+    float *all_s = (float *)malloc(sizeof(float) * n_ranges * nq * k);
+    uint64_t *all_i = (uint64_t *)malloc(sizeof(uint64_t) * n_ranges * nq * k);
+    size_t *all_sz = (size_t *)calloc(n_ranges * nq, sizeof(size_t));
+    const long long n_tiles = (long long)(n_ranges * n_groups);
+#pragma omp parallel for schedule(dynamic, 1) num_threads(n_threads)
+    for (long long t = 0; t < n_tiles; t++) {
+        const size_t r = (size_t)t / n_groups, q0 = ((size_t)t % n_groups) * TVO_NQ;
+        const size_t b0 = r * stride, b1 = b0 + stride < n_blocks ? b0 + stride : n_blocks;
+        heap_t heaps[TVO_NQ];
+        const int nqm = (int)(nq - q0 < TVO_NQ ? nq - q0 : TVO_NQ);
+        const int8_t *w8[TVO_NQ];
+        for (int j = 0; j < nqm; j++) {
+            w8[j] = W + (q0 + (size_t)j) * (size_t)dim;
+            heaps[j].hs = all_s + (r * nq + q0 + (size_t)j) * k;
+            heaps[j].hi = all_i + (r * nq + q0 + (size_t)j) * k;
+            heaps[j].sz = 0; heaps[j].mi = 0; heaps[j].mn = -INFINITY;
+        }
+        scan_range_vnni(vm_codes, G, b0, b1, n, w8, zero + q0, qscale + q0, qbias + q0, nqm, levels,
+                        vec_scales, mask, heaps, k);
+        for (int j = 0; j < nqm; j++) all_sz[r * nq + q0 + (size_t)j] = heaps[j].sz;
+    }
+    int err = 0;
+#pragma omp parallel for schedule(static) num_threads(n_threads)
+    for (long long qi = 0; qi < (long long)nq; qi++) {
+        pair_t *pairs = (pair_t *)malloc(sizeof(pair_t) * n_ranges * k);
+        size_t np = 0;
+        for (size_t r = 0; r < n_ranges; r++) {
+            size_t sz = all_sz[r * nq + (size_t)qi];
+            for (size_t j = 0; j < sz; j++) {
+                pairs[np].s = all_s[(r * nq + (size_t)qi) * k + j];
+                pairs[np].i = all_i[(r * nq + (size_t)qi) * k + j];
+                np++;
+            }
+        }
+        qsort(pairs, np, sizeof(pair_t), cmp_pair);          /* search.rs:4279-4298 */
+        if (np < k) {
+#pragma omp atomic write
+            err = 1;
+        }
+        for (size_t j = 0; j < k && j < np; j++) {
+            out_scores[(size_t)qi * k + j] = pairs[j].s;
+            out_indices[(size_t)qi * k + j] = (int64_t)pairs[j].i;
+        }
+        free(pairs);
+    }
+    free(all_s); free(all_i); free(all_sz); free(qscale); free(qbias); free(W); free(zero);
+    return err ? TVO_ERR_BAD_ARGUMENT : TVO_OK;
+#else
+    (void)queries; (void)nq; (void)rot; (void)vm_codes; (void)centroids; (void)vec_scales; (void)dim; (void)n; (void)k;
+    (void)mask; (void)out_scores; (void)out_indices; (void)out_k_eff; (void)n_threads;
+    return TVO_ERR_BAD_ARGUMENT;
+#endif
+}
+
+/* ======================================================================= */
 /* Fixture helpers                                                          */
 /* ======================================================================= */
 

@@ -21,6 +21,8 @@
  *                            incomplete beta function, conditional means in closed
  *                            form, no quadrature) reproduces the golden hashes and
  *                            equals this function bit for bit in every cell.
+ *   tvo_search_fast,         equality with tvo_search on the same inputs (tests).
+ *   tvo_search_vnni
  *   tvo_fit_calibration,
  *   tvo_encode, tvo_norm     pinned: calibration/codes/scales hashes, 8 cells.
  *   tvo_repack_seq et al.    pinned: closed-form byte maps (src/pack.rs:964-1008).
@@ -175,6 +177,20 @@ int tvo_search(int mode, const float *queries, size_t nq, const tvo_rotation *ro
 int tvo_search_fast(const float *queries, size_t nq, const tvo_rotation *rot,
                     const uint8_t *seq_codes, const float *centroids, const float *vec_scales,
                     int bits, int dim, size_t n, size_t k, const uint64_t *mask_words,
+                    float *out_scores, int64_t *out_indices, size_t *out_k_eff, int n_threads);
+
+/* The reference's production path for 4-bit on an AVX-512 VNNI host (search.rs:1392-1567):
+ * vpshufb level lookup + vpdpbusd over the vector-major layout (pack.rs:1269-1271), eight
+ * queries per pass over a block.  tvo_seq_to_vector_major builds that layout (what the
+ * reference keeps at rest, pack.rs:1347-1358); tvo_search_vnni answers exactly as tvo_search
+ * mode P does (tests compare bit for bit) and returns TVO_ERR_BAD_ARGUMENT on a host without
+ * the instructions (tvo_have_vnni() == 0).  Uncalibrated indexes, k <= 1024.  This is what the
+ * CPU-baseline timing runs where it can. */
+int tvo_have_vnni(void);
+int tvo_seq_to_vector_major(const uint8_t *seq, size_t n, int bits, int dim, uint8_t *vm);
+int tvo_search_vnni(const float *queries, size_t nq, const tvo_rotation *rot,
+                    const uint8_t *vm_codes, const float *centroids, const float *vec_scales,
+                    int dim, size_t n, size_t k, const uint64_t *mask_words,
                     float *out_scores, int64_t *out_indices, size_t *out_k_eff, int n_threads);
 
 /* Caller-side checks that precede the seam (turbovec/src/lib.rs:1363-1380,

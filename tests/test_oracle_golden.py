@@ -433,3 +433,35 @@ def test_search_fast_equals_search(oracle, dim, bits, n):
     s, i = O.search(rot, seq, scales, q, 10, bits, dim, n, mask_words=words)
     s2, i2 = O.search_fast(rot, seq, scales, q, 10, bits, dim, n, mask_words=words, n_threads=3)
     assert np.array_equal(i, i2) and _eq_bits(s, s2)
+
+
+# The reference's AVX-512 VNNI production kernel, restated (search.rs:1392-1567 over the vector-major
+# layout, pack.rs:1269-1271): same slots and score bits as the scalar statement of mode P, ragged last
+# block, masks, fewer than eight queries in the last group, ties.  Skipped on a host without VNNI.
+@pytest.mark.parametrize("dim,n,nq", [(1536, 3003, 37), (128, 5003, 9), (768, 70, 3), (64, 32, 8)])
+def test_search_vnni_equals_search(oracle, dim, n, nq):
+    O = oracle
+    if not O.have_vnni():
+        pytest.skip("host has no AVX-512 VNNI")
+    rng = np.random.default_rng(23)
+    v = rng.standard_normal((n, dim)).astype(np.float32)
+    v[n // 2] = v[n // 3]                                   # a duplicate row: equal scores, lower slot first
+    q = rng.standard_normal((nq, dim)).astype(np.float32)
+    rot = O.Rotation(dim)
+    packed, scales = O.encode(rot, v, 4)
+    seq = O.repack_seq(packed, n, 4, dim)
+    vm = O.seq_to_vector_major(seq, n, 4, dim)
+    # layout: byte of (block b, group g, lane l) sits at b*G*32 + (g/4)*128 + (l/16)*64 + (l%16)*4 + g%4
+    G = dim // 2
+    for (b, g, l) in [(0, 0, 0), (0, 5, 17), ((n - 1) // 32, G - 1, (n - 1) % 32), (1 % ((n + 31) // 32), 6, 31)]:
+        assert vm[b * G * 32 + (g // 4) * 128 + (l // 16) * 64 + (l % 16) * 4 + g % 4] == seq[(b * G + g) * 32 + l]
+    for k in (1, 10, 64):
+        s, i = O.search(rot, seq, scales, q, k, 4, dim, n, mode=O.MODE_P)
+        for threads in (1, 5):
+            s2, i2 = O.search_vnni(rot, vm, scales, q, k, dim, n, n_threads=threads)
+            assert np.array_equal(i, i2) and _eq_bits(s, s2)
+    for frac in (0.5, 0.03):
+        words, _ = O.pack_mask(rng.random(n) < frac)
+        s, i = O.search(rot, seq, scales, q, 10, 4, dim, n, mask_words=words, mode=O.MODE_P)
+        s2, i2 = O.search_vnni(rot, vm, scales, q, 10, dim, n, mask_words=words, n_threads=3)
+        assert np.array_equal(i, i2) and _eq_bits(s, s2)
