@@ -59,7 +59,8 @@ def parse():
     ap.add_argument("--cpu-sample", type=int, default=2_000_000, help="vectors in the CPU-baseline sample (0 = skip)")
     ap.add_argument("--cpu-threads", type=int, default=16)
     ap.add_argument("--no-config3", action="store_true",
-                    help="skip the extra key for configuration 3 (10M x 1536 2-bit, k=100, batches 1 and 1024)")
+                    help="skip the extra keys: configuration 3 (10M x 1536 2-bit, k=100, batches 1 and 1024) and the "
+                         "adversarial insertion orders")
     ap.add_argument("--copy-probe", action="store_true",
                     help="only run the plain copy kernel over a 4 GiB buffer (counter calibration) and exit")
     return ap.parse_args()
@@ -156,6 +157,75 @@ def config3_extra(T, torch, build_index, run, args):
     res["overflow_redos"] = ix.overflow_redos()
     ix.close()
     return res
+
+
+def adversarial_extra(T, torch, run, args, normal_ms):
+    """What the candidate-overflow path costs at full size (10M x 1536 4-bit, k=10, 1024 queries) on
+    two insertion orders chosen against it.  (1) a 1000-cluster mixture inserted cluster by cluster,
+    queries next to database rows: every query has thousands of near neighbours in a few hundred
+    consecutive blocks.  (2) an index laid out against the sampler itself: every block the sampling
+    levels of the first pass read (multiples of the level strides) holds rows pointing away from
+    the queries, every other block rows pointing towards them, so the first pass's floors are far
+    too low and every query overflows.  Overflowed queries are scanned once more together (ladder
+    shifted half a stride, from raised floors); what still overflows goes to the exact path."""
+    dev = torch.device("cuda:0")
+    n, dim, k, nq = 10_000_000, 1536, 10, 1024
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(7)
+    out = {"normal_ms_per_step": normal_ms}
+
+    def timed(ix, q, steps=3):
+        torch.cuda.synchronize()
+        os_ = torch.empty(nq, k, device=dev)
+        oi = torch.empty(nq, k, dtype=torch.int64, device=dev)
+        ix.search_dev(q.data_ptr(), nq, k, os_.data_ptr(), oi.data_ptr())
+        r0, e0 = ix.overflow_redos(), ix.exact_redos()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            ix.search_dev(q.data_ptr(), nq, k, os_.data_ptr(), oi.data_ptr())
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+        return {"ms_per_step": ms, "vs_normal": ms / normal_ms,
+                "queries_repeated_per_step": (ix.overflow_redos() - r0) / steps,
+                "queries_on_exact_path_per_step": (ix.exact_redos() - e0) / steps}
+
+    # (1) clustered, cluster by cluster
+    centres = torch.randn(1000, dim, device=dev, generator=gen)
+    ix = T.NativeIndex(dim, 4)
+    keep = None
+    for c0 in range(0, n, 100_000):
+        cid = torch.arange(c0, c0 + 100_000, device=dev) // 10_000
+        v = centres[cid] + 0.3 * torch.randn(100_000, dim, device=dev, generator=gen)
+        v = (v / v.norm(dim=1, keepdim=True)).contiguous()
+        if keep is None:
+            keep = v[:: 100_000 // nq][:nq].clone()
+        torch.cuda.synchronize()
+        ix.add_dev(v.data_ptr(), v.shape[0])
+    q = keep + 0.05 * torch.randn(nq, dim, device=dev, generator=gen) / dim ** 0.5
+    q = (q / q.norm(dim=1, keepdim=True)).contiguous()
+    out["clustered_inserted_cluster_by_cluster"] = timed(ix, q)
+    ix.close()
+    del ix, v, centres
+    torch.cuda.empty_cache()
+
+    # (2) against the sampler: strides of the first pass's sampling levels at this size
+    u = torch.randn(dim, device=dev, generator=gen)
+    u = u / u.norm()
+    ix = T.NativeIndex(dim, 4)
+    for c0 in range(0, n, 100_000):
+        blocks = torch.arange(c0, c0 + 100_000, device=dev) // 32
+        sampled = (blocks % 98 == 0) | (blocks % 9765 == 0)
+        sign = torch.where(sampled, -1.0, 1.0).unsqueeze(1)
+        v = sign * 0.3 * u + torch.randn(100_000, dim, device=dev, generator=gen) / dim ** 0.5
+        v = (v / v.norm(dim=1, keepdim=True)).contiguous()
+        torch.cuda.synchronize()
+        ix.add_dev(v.data_ptr(), v.shape[0])
+    q = u + 0.5 * torch.randn(nq, dim, device=dev, generator=gen) / dim ** 0.5
+    q = (q / q.norm(dim=1, keepdim=True)).contiguous()
+    out["laid_out_against_the_sampler"] = timed(ix, q)
+    ix.close()
+    return out
 
 
 def main():
@@ -320,11 +390,14 @@ def main():
     # queries of the timed steps that left the sampled path for the exact one (candidate overflow);
     # Gaussian rows never do, and a non-zero count would mean the timed steps include that path's cost
     out["overflow_redos"] = ix.overflow_redos()
+    out["exact_redos"] = ix.exact_redos()
     if not args.no_config3 and (n, dim, bits) == (10_000_000, 1536, 4) and not args.tile_groups:
         ix.close()
         del ix
         torch.cuda.empty_cache()
         out["config3"] = config3_extra(T, torch, build_index, run, args)
+        torch.cuda.empty_cache()
+        out["adversarial"] = adversarial_extra(T, torch, run, args, out["ms_per_step"])
     if args.cpu_sample > 0:
         out["cpu_baseline"] = cpu_baseline(args)
     print(json.dumps(out))

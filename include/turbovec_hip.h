@@ -227,9 +227,11 @@ int tv_debug_queries_per_launch(const tv_index *ix, int *queries);
  * instead of the batched ones; bit 2 keeps them off the all-queries-per-pass
  * kernel only. */
 int tv_debug_set_path(tv_index *ix, int force_full_lists);
-/* How many queries so far had to be redone through that path because their
- * candidate buffer overflowed. */
+/* How many queries so far did not finish in the single sampled pass because their
+ * candidate buffer overflowed (they are scanned once more, all together, from a raised
+ * floor), and how many of those went on to the exact list / select path. */
 int tv_debug_overflow_redos(const tv_index *ix, size_t *count);
+int tv_debug_exact_redos(const tv_index *ix, size_t *count);
 /* Bandwidth probe on the index's stream: reps launches of a pure read-sum over
  * d_src (d_dst NULL) or of a plain copy d_src -> d_dst, bytes each; mean
  * milliseconds per launch.  Calibrates the achievable HBM rate and gives the

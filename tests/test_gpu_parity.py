@@ -474,8 +474,8 @@ def test_sampled_path_matches_oracle_and_full_path(T, oracle, bits, mode):
 def test_candidate_overflow_is_redone_exactly(T, oracle):
     """An index ordered against the sampler: every block the sampling pass reads
     holds poor matches and all the others hold near-duplicates of the query, so
-    the floor is low, the candidate buffer overflows, and the query is redone
-    through the full list path with the same exact answer."""
+    the floor is low, the candidate buffer overflows, and the query is scanned
+    once more from a raised floor, with the same exact answer."""
     O = oracle
     dim, bits, n = 64, 4, 64 * 32 * 24
     rng = np.random.default_rng(8)
@@ -490,6 +490,9 @@ def test_candidate_overflow_is_redone_exactly(T, oracle):
     os_, oi = oidx.search(q, 10)
     assert np.array_equal(i, oi) and bits_equal(s, os_)
     assert ix.overflow_redos() >= 1
+    # the repeated pass samples other blocks (half a stride in) and starts from the raised floor:
+    # it settles the query without the exact path
+    assert ix.exact_redos() == 0
     ix.close()
 
 

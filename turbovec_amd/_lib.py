@@ -33,6 +33,7 @@ EXPORTS = [
     "tv_debug_stream_probe", "tv_debug_mfma_probe", "tv_debug_set_path", "tv_debug_overflow_redos",
     "tv_host_snapshot_len", "tv_host_snapshot_compose", "tv_host_snapshot_info", "tv_host_snapshot_extract",
     "tv_index_to_bytes", "tv_index_from_bytes", "tv_search_dev_noalloc", "tv_noalloc_scratch_bytes",
+    "tv_debug_exact_redos",
 ]
 
 _lib = None
@@ -98,6 +99,7 @@ def lib():
     L.tv_index_device_ptrs.argtypes = [vp, C.POINTER(vp), C.POINTER(vp), C.POINTER(sz)]
     L.tv_debug_set_path.argtypes = [vp, i32]
     L.tv_debug_overflow_redos.argtypes = [vp, C.POINTER(sz)]
+    L.tv_debug_exact_redos.argtypes = [vp, C.POINTER(sz)]
     L.tv_debug_stream_probe.argtypes = [vp, vp, vp, sz, i32, C.POINTER(C.c_float)]
     L.tv_debug_mfma_probe.argtypes = [vp, i32, i32, C.POINTER(C.c_float), C.POINTER(C.c_double)]
     L.tv_host_rotation_tables.argtypes = [i32, vp, vp, C.POINTER(i32), C.POINTER(C.c_float)]
@@ -302,6 +304,11 @@ class NativeIndex:
     def overflow_redos(self):
         c = C.c_size_t(0)
         check(lib().tv_debug_overflow_redos(self.h, C.byref(c)))
+        return c.value
+
+    def exact_redos(self):
+        c = C.c_size_t(0)
+        check(lib().tv_debug_exact_redos(self.h, C.byref(c)))
         return c.value
 
     def mfma_probe(self, iters=2000, reps=3):

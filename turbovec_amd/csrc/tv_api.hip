@@ -300,6 +300,24 @@ SampledPlan sampled_plan(const tv_index *ix, size_t cq) {
     return p;
 }
 
+// What a chunk keeps at the head of the workspace across its passes: raised floors, the rows to
+// repeat, and their queries packed.
+size_t redo_header_bytes(const tv_index *ix, size_t cq) {
+    return 2 * round_up(cq * 4, 256) + round_up(cq * size_t(ix->geo.dim) * 4, 256);
+}
+
+// Workspace a chunk of cq queries may need on the sampled path: its own pass, or the repeated
+// pass over a smaller packed batch that falls to another kernel with more candidate segments.
+// Workspace a chunk of cq queries needs on the sampled path: its own pass, and room for the
+// repeated pass to run at least a tile of queries at a time (a smaller packed batch may fall to
+// another kernel with more candidate segments per query; it is then cut into pieces that fit).
+constexpr size_t kRepeatPieces[] = {1024, 512, 256, 128, 96, 64, 32};
+size_t sampled_need_worst(const tv_index *ix, size_t cq) {
+    size_t need = sampled_plan(ix, cq).need;
+    need = std::max(need, sampled_plan(ix, std::min<size_t>(cq, tv::kQTile)).need);
+    return need + redo_header_bytes(ix, cq);
+}
+
 // Full-range search without sampling: per-lane lists with shared thresholds for
 // k <= 32, dense scores + radix select beyond.  Always exact; used for the
 // queries whose candidate buffer overflowed and for very large k.
@@ -453,89 +471,154 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
 
     for (size_t q0 = 0; q0 < nq; q0 += kChunkQueries) {
         const size_t cq = std::min(kChunkQueries, nq - q0);
-        const SampledPlan plan = sampled_plan(ix, cq);
-        const size_t tile_q = plan.tile_q, n_tiles = plan.n_tiles, cq_pad = plan.cq_pad, seg_stride = plan.seg_stride;
-        const bool wide = plan.wide;
-        const int grid = plan.grid;
-        rc = ensure_workspace(ix, plan.need);
+        const float *d_q = d_queries + q0 * g.dim;
+        float *d_os = d_out_scores + q0 * k_eff;
+        int64_t *d_oi = d_out_idx + q0 * k_eff;
+        // sized for the repeated pass too: the head of the workspace must survive between the passes
+        rc = ensure_workspace(ix, sampled_need_worst(ix, cq));
         if (rc != TV_OK) return rc;
-        Arena ar;
-        ar.base = static_cast<uint8_t *>(ix->ws);
-        Prepared pq;
-        size_t n_timed = 0;
-        rc = prepare_queries(ix, ar, d_queries + q0 * g.dim, cq, pq);
-        if (rc != TV_OK) return rc;
-        int *d_tau = ar.take<int>(n_tiles * tv::kQTile);
-        uint64_t *d_cand = ar.take<uint64_t>(cq_pad * seg_stride * tv::kSegCap);
-        uint32_t *d_cnt = ar.take<uint32_t>(cq_pad * seg_stride);
-        uint32_t *d_over = ar.take<uint32_t>(cq_pad);
-        // no per-search clears: the first level reads the index's standing array of open floors,
-        // every later one the floors k_final wrote, and k_final writes every overflow flag
+        Arena head;
+        head.base = static_cast<uint8_t *>(ix->ws);
+        int *d_raise = head.take<int>(cq);
+        uint32_t *d_rows = head.take<uint32_t>(cq);
+        float *d_redo_q = head.take<float>(cq * g.dim);
 
-        const int nt_batched = (mode_p && cq > size_t(tv::kQTile) && !ix->no_batched) ? tv::batched_tiles(g.nch) : 0;
-        const int bgrid = tv::batched_grid_blocks(ix->device, g.nch);
-        for (size_t lv = 0; lv < steps.size(); ++lv) {
-            const bool last = lv + 1 == steps.size();
-            const size_t level_blocks = (n_blocks + steps[lv] - 1) / steps[lv];
-            // level 1 appends every slot it reads: two blocks per workgroup fill a segment exactly
-            const int lgrid = int(std::min<size_t>(size_t(grid), std::max<size_t>(1, (level_blocks + 1) / 2)));
-            const bool batched = nt_batched > 0 && !wide;
-            const size_t tiles_per_launch = wide ? n_tiles : batched ? size_t(nt_batched) : 1;
-            ix->last_queries_per_launch = int(std::min(cq, tile_q * tiles_per_launch));
-            int n_seg = lgrid;
-            size_t launch_no = 0;
-            for (size_t t = 0; t < n_tiles; t += tiles_per_launch, ++launch_no) {
-                tv::ScanArgs a;
-                fill_scan_args(ix, a);
-                a.mask = d_mask;
-                a.tables = pq.d_tables + t * (mode_p ? pq.table_bytes_per_tile : tile_q * size_t(g.nch) * 1024);
-                a.qscale = pq.d_qscale + t * tile_q;
-                a.qbias = pq.d_qbias + t * tile_q;
-                a.nq_tile = int(std::min<size_t>(tile_q * tiles_per_launch, cq - t * tile_q));
-                a.k = 1;
-                a.gtau = (lv == 0 ? ix->d_tau_open : d_tau) + t * tv::kQTile;
-                a.b_step = steps[lv];
-                a.cand = d_cand + t * tile_q * seg_stride * tv::kSegCap;
-                a.cand_cnt = d_cnt + t * tile_q * seg_stride;
-                a.seg_stride = uint32_t(seg_stride);
-                const bool timed = timing && last && int(launch_no) < kMaxTimedTiles;
-                if (timed) TV_HIP(hipEventRecord(ix->ev_start[launch_no], ix->stream));
-                if (wide) {
-                    n_seg = grid;
-                    TV_HIP(tv::launch_scan_p4_wide(a, n_seg, ix->stream));
-                } else if (batched) {
-                    n_seg = int(std::min<size_t>(size_t(bgrid), seg_stride));
-                    TV_HIP(tv::launch_scan_p4_batched(a, n_seg, ix->stream));
-                } else if (mode_p) {
-                    TV_HIP(tv::launch_scan_p4(a, lgrid, tv::kModeAppend, ix->stream));
-                } else {
-                    TV_HIP(tv::launch_scan_lut(a, lgrid, tv::kModeAppend, ix->stream));
+        // One pass over `pq_n` queries: the ladder from open floors, or, for the packed batch of
+        // queries to repeat, the ladder again from the floors the pass before raised for them.
+        auto pass = [&](size_t row0, size_t pq_n, bool repeat) -> int {
+            const SampledPlan plan = sampled_plan(ix, pq_n);
+            const size_t tile_q = plan.tile_q, n_tiles = plan.n_tiles, cq_pad = plan.cq_pad, seg_stride = plan.seg_stride;
+            const bool wide = plan.wide;
+            const int grid = plan.grid;
+            int prc = ensure_workspace(ix, head.used + plan.need);
+            if (prc != TV_OK) return prc;
+            Arena ar;
+            ar.base = static_cast<uint8_t *>(ix->ws) + head.used;
+            int *d_tau = ar.take<int>(n_tiles * tv::kQTile);
+            if (repeat)
+                TV_HIP(tv::launch_gather_redo(d_q, d_rows + row0, d_raise, g.dim, int(tile_q), pq_n, d_redo_q, d_tau, ix->stream));
+            Prepared pq;
+            size_t n_timed = 0;
+            prc = prepare_queries(ix, ar, repeat ? d_redo_q : d_q, pq_n, pq);
+            if (prc != TV_OK) return prc;
+            uint64_t *d_cand = ar.take<uint64_t>(cq_pad * seg_stride * tv::kSegCap);
+            uint32_t *d_cnt = ar.take<uint32_t>(cq_pad * seg_stride);
+            uint32_t *d_over = ar.take<uint32_t>(cq_pad);
+            // no per-search clears: the first level reads the index's standing array of open floors,
+            // every later one the floors k_final wrote, and k_final writes every overflow flag
+
+            const int nt_batched = (mode_p && pq_n > size_t(tv::kQTile) && !ix->no_batched) ? tv::batched_tiles(g.nch) : 0;
+            const int bgrid = tv::batched_grid_blocks(ix->device, g.nch);
+            for (size_t lv = 0; lv < steps.size(); ++lv) {
+                const bool last = lv + 1 == steps.size();
+                // A repeated pass samples other blocks than the pass that misjudged the floor: its
+                // sampling levels start half a stride in (an even number of blocks, so that mask
+                // words stay aligned).  Sampling levels only yield floors, never slots, so the
+                // shifted origin needs no correction downstream.
+                const uint32_t off = (repeat && steps[lv] >= 4) ? (steps[lv] / 2) & ~1u : 0u;
+                const size_t level_blocks = (n_blocks - off + steps[lv] - 1) / steps[lv];
+                // level 1 appends every slot it reads: two blocks per workgroup fill a segment exactly
+                const int lgrid = int(std::min<size_t>(size_t(grid), std::max<size_t>(1, (level_blocks + 1) / 2)));
+                const bool batched = nt_batched > 0 && !wide;
+                const size_t tiles_per_launch = wide ? n_tiles : batched ? size_t(nt_batched) : 1;
+                if (!repeat) ix->last_queries_per_launch = int(std::min(pq_n, tile_q * tiles_per_launch));
+                int n_seg = lgrid;
+                size_t launch_no = 0;
+                for (size_t t = 0; t < n_tiles; t += tiles_per_launch, ++launch_no) {
+                    tv::ScanArgs a;
+                    fill_scan_args(ix, a);
+                    a.mask = d_mask;
+                    a.tables = pq.d_tables + t * (mode_p ? pq.table_bytes_per_tile : tile_q * size_t(g.nch) * 1024);
+                    a.qscale = pq.d_qscale + t * tile_q;
+                    a.qbias = pq.d_qbias + t * tile_q;
+                    a.nq_tile = int(std::min<size_t>(tile_q * tiles_per_launch, pq_n - t * tile_q));
+                    a.k = 1;
+                    a.gtau = ((lv == 0 && !repeat) ? ix->d_tau_open : d_tau) + t * tv::kQTile;
+                    a.b_step = steps[lv];
+                    if (off) {
+                        a.codes += size_t(off) * g.block_bytes();
+                        a.scales += size_t(off) * tv::kVecBlock;
+                        if (a.mask) a.mask += off / 2;
+                        a.n_blocks -= off;
+                        a.n -= off * tv::kVecBlock;
+                    }
+                    a.cand = d_cand + t * tile_q * seg_stride * tv::kSegCap;
+                    a.cand_cnt = d_cnt + t * tile_q * seg_stride;
+                    a.seg_stride = uint32_t(seg_stride);
+                    const bool timed = timing && !repeat && last && int(launch_no) < kMaxTimedTiles;
+                    if (timed) TV_HIP(hipEventRecord(ix->ev_start[launch_no], ix->stream));
+                    if (wide) {
+                        n_seg = grid;
+                        TV_HIP(tv::launch_scan_p4_wide(a, n_seg, ix->stream));
+                    } else if (batched) {
+                        n_seg = int(std::min<size_t>(size_t(bgrid), seg_stride));
+                        TV_HIP(tv::launch_scan_p4_batched(a, n_seg, ix->stream));
+                    } else if (mode_p) {
+                        TV_HIP(tv::launch_scan_p4(a, lgrid, tv::kModeAppend, ix->stream));
+                    } else {
+                        TV_HIP(tv::launch_scan_lut(a, lgrid, tv::kModeAppend, ix->stream));
+                    }
+                    if (timed) TV_HIP(hipEventRecord(ix->ev_stop[launch_no], ix->stream));
                 }
-                if (timed) TV_HIP(hipEventRecord(ix->ev_stop[launch_no], ix->stream));
+                if (last && timing && !repeat) n_timed = std::min<size_t>(launch_no, size_t(kMaxTimedTiles));
+                // the first final pass may hand raised floors to a repeated one; the repeated pass
+                // sends what still does not fit to the exact path
+                TV_HIP(tv::launch_final(d_cand, d_cnt, uint32_t(n_seg), uint32_t(seg_stride), int(k_eff), int(k_floor),
+                                        int(pq_n), d_os, d_oi, d_over, last ? nullptr : d_tau, int(tile_q), (lv > 0 || repeat) ? 1 : 0,
+                                        (last && !repeat) ? d_raise : nullptr, repeat ? d_rows + row0 : nullptr, ix->stream));
             }
-            if (last && timing) n_timed = std::min<size_t>(launch_no, size_t(kMaxTimedTiles));
-            TV_HIP(tv::launch_final(d_cand, d_cnt, uint32_t(n_seg), uint32_t(seg_stride), int(k_eff), int(k_floor),
-                                    int(cq), d_out_scores + q0 * k_eff, d_out_idx + q0 * k_eff, d_over,
-                                    last ? nullptr : d_tau, int(tile_q), lv > 0 ? 1 : 0, ix->stream));
+            TV_HIP(hipMemcpyAsync(h_over, d_over, pq_n * sizeof(uint32_t), hipMemcpyDeviceToHost, ix->stream));
+            TV_HIP(hipStreamSynchronize(ix->stream));
+            for (size_t t = 0; t < n_timed; ++t) {
+                float ms = 0.0f;
+                TV_HIP(hipEventElapsedTime(&ms, ix->ev_start[t], ix->ev_stop[t]));
+                ix->last_scan_ms += ms;
+                ix->last_scan_launches += 1;
+            }
+            return TV_OK;
+        };
+
+        rc = pass(0, cq, false);
+        if (rc != TV_OK) return rc;
+        // Queries whose candidates did not fit (an unlucky sample, adversarial order).  Those that
+        // came back with a raised floor (flag 1) are packed and scanned once more, all together;
+        // what still does not fit then, and what had no floor to raise (flag 2), is redone exactly.
+        uint32_t rows[kChunkQueries];
+        size_t n_rows = 0, n_exact = 0;
+        uint32_t exact_rows[kChunkQueries];
+        for (size_t q = 0; q < cq; ++q) {
+            if (h_over[q] == 1u) rows[n_rows++] = uint32_t(q);
+            else if (h_over[q] != 0u) exact_rows[n_exact++] = uint32_t(q);
         }
-        TV_HIP(hipMemcpyAsync(h_over, d_over, cq * sizeof(uint32_t), hipMemcpyDeviceToHost, ix->stream));
-        TV_HIP(hipStreamSynchronize(ix->stream));
-        for (size_t t = 0; t < n_timed; ++t) {
-            float ms = 0.0f;
-            TV_HIP(hipEventElapsedTime(&ms, ix->ev_start[t], ix->ev_stop[t]));
-            ix->last_scan_ms += ms;
-            ix->last_scan_launches += 1;
+        ix->overflow_redos += n_rows + n_exact;
+        if (n_rows) {
+            std::memcpy(h_over, rows, n_rows * sizeof(uint32_t));   // pinned staging for the upload
+            TV_HIP(hipMemcpyAsync(d_rows, h_over, n_rows * sizeof(uint32_t), hipMemcpyHostToDevice, ix->stream));
+            TV_HIP(hipStreamSynchronize(ix->stream));
+            // all of them in one pass when the workspace holds that pass, else in the largest pieces it holds
+            const size_t room = ix->ws_bytes - head.used;
+            for (size_t r0 = 0; r0 < n_rows;) {
+                size_t piece = std::min<size_t>(n_rows - r0, tv::kQTile);
+                for (size_t cand_piece : kRepeatPieces) {
+                    const size_t m = std::min(cand_piece, n_rows - r0);
+                    if (sampled_plan(ix, m).need <= room) { piece = m; break; }
+                }
+                rc = pass(r0, piece, true);
+                if (rc != TV_OK) return rc;
+                for (size_t r = 0; r < piece; ++r)
+                    if (h_over[r] != 0u) exact_rows[n_exact++] = rows[r0 + r];
+                r0 += piece;
+            }
         }
-        // queries whose candidates did not fit (an unlucky sample, adversarial order): redo exactly
-        for (size_t qa = 0; qa < cq;) {
-            if (!h_over[qa]) { ++qa; continue; }
-            size_t qb = qa;
-            while (qb < cq && h_over[qb]) ++qb;
-            ix->overflow_redos += qb - qa;
-            rc = search_robust(ix, d_queries + (q0 + qa) * g.dim, qb - qa, k_eff, d_mask,
-                               d_out_scores + (q0 + qa) * k_eff, d_out_idx + (q0 + qa) * k_eff, false);
+        std::sort(exact_rows, exact_rows + n_exact);
+        ix->exact_redos += n_exact;
+        for (size_t i = 0; i < n_exact;) {
+            size_t e = i + 1;
+            while (e < n_exact && exact_rows[e] == exact_rows[e - 1] + 1) ++e;     // runs of neighbours go together
+            const size_t qa = exact_rows[i], cnt = e - i;
+            rc = search_robust(ix, d_q + qa * g.dim, cnt, k_eff, d_mask, d_os + qa * k_eff, d_oi + qa * k_eff, false);
             if (rc != TV_OK) return rc;
-            qa = qb;
+            i = e;
         }
     }
     return TV_OK;
@@ -966,7 +1049,7 @@ int tv_search_dev_noalloc(tv_index *ix, const float *d_queries, size_t nq, size_
     if (k_eff != 0 && nq != 0) {
         const size_t cq = std::min(nq, kChunkQueries);
         need = robust_need(ix, cq, k_eff);
-        if (k_eff <= size_t(tv::kMaxSampledK) && !ix->force_robust) need = std::max(need, sampled_plan(ix, cq).need);
+        if (k_eff <= size_t(tv::kMaxSampledK) && !ix->force_robust) need = std::max(need, sampled_need_worst(ix, cq));
     }
     if (need > kScratchBytes) {
         g_last_error = "tv_search_dev_noalloc: " + std::to_string(nq) + " queries, k=" + std::to_string(k) + " over " +
@@ -1276,6 +1359,12 @@ int tv_debug_set_path(tv_index *ix, int force_full_lists) {
 int tv_debug_overflow_redos(const tv_index *ix, size_t *count) {
     if (!ix || !count) return TV_ERR_BAD_ARGUMENT;
     *count = ix->overflow_redos;
+    return TV_OK;
+}
+
+int tv_debug_exact_redos(const tv_index *ix, size_t *count) {
+    if (!ix || !count) return TV_ERR_BAD_ARGUMENT;
+    *count = ix->exact_redos;
     return TV_OK;
 }
 

@@ -122,10 +122,16 @@ hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, cons
 // emits the k_eff best (tau_out == nullptr; a query that did not fit is flagged in overflow) or, for a
 // sampling level, writes the order key of the k_floor-th best as the query's next floor to
 // tau_out[(q / tau_stride_q) * kQTile + q % tau_stride_q] (keep_floor: a level that gathers fewer than k_eff
-// candidates leaves the floor already there in place instead of opening it).
+// candidates leaves the floor already there in place instead of opening it).  A final pass that
+// overflows writes flag 1 and a raised floor to raise_out[q] when raise_out is given (flag 2 and
+// nothing otherwise); row_map, when given, names the output row of each query.
 hipError_t launch_final(const uint64_t *cand, const uint32_t *cand_cnt, uint32_t n_seg, uint32_t seg_stride,
                         int k_eff, int k_floor, int nq, float *out_scores, int64_t *out_idx, uint32_t *overflow,
-                        int *tau_out, int tau_stride_q, int keep_floor, hipStream_t s);
+                        int *tau_out, int tau_stride_q, int keep_floor, int *raise_out, const uint32_t *row_map,
+                        hipStream_t s);
+// Packs the queries rows[0..n_redo) of a chunk and their raised floors for one more full scan.
+hipError_t launch_gather_redo(const float *d_q, const uint32_t *d_rows, const int *d_raised, int dim, int tile_q,
+                              size_t n_redo, float *d_q_out, int *d_tau_out, hipStream_t s);
 hipError_t launch_fill_i32(int *p, int v, size_t n, hipStream_t s);
 hipError_t launch_probe(const void *src, void *dst, size_t bytes, int copy, uint32_t *sink, hipStream_t s);
 hipError_t launch_probe_mfma(int device, int iters, uint32_t *sink, double *ops, hipStream_t s);
@@ -169,7 +175,8 @@ struct tv_index {
     size_t ws_bytes = 0;
     bool ws_fixed = false;         // ws is a lent buffer of fixed size (tv_search_dev_noalloc): never reallocated
     void *scratch = nullptr;       // this device's copy of the library's static scratch array
-    uint32_t *h_flags = nullptr;   // pinned host memory: the overflow flags of one chunk of queries
+    uint32_t *h_flags = nullptr;   // pinned host memory: the overflow flags of one chunk of queries, then the rows to repeat
+    size_t exact_redos = 0;        // queries that went on to the exact path
     float last_scan_ms = 0.0f;
     int last_scan_launches = 0;
     int last_queries_per_launch = 0;   // queries one full-scan launch of the last search served

@@ -97,6 +97,17 @@ __global__ void k_move_lane(uint8_t *__restrict__ nat, float *__restrict__ scale
     }
 }
 
+// Queries whose candidates overflowed, packed for one more full scan: row r of the packed batch
+// is query rows[r] of the chunk, its floor the raised one k_final left for it, placed where the
+// scan kernels read the floors of tile r / tile_q.
+__global__ __launch_bounds__(256) void k_gather_redo(const float *__restrict__ q, const uint32_t *__restrict__ rows,
+                                                     const int *__restrict__ raised, int dim, int tile_q,
+                                                     float *__restrict__ q_out, int *__restrict__ tau_out) {
+    const uint32_t r = blockIdx.x, o = rows[r];
+    for (int i = threadIdx.x; i < dim; i += 256) q_out[size_t(r) * dim + i] = q[size_t(o) * dim + i];
+    if (threadIdx.x == 0) tau_out[(r / tile_q) * kQTile + r % tile_q] = raised[o];
+}
+
 __global__ void k_fill_i32(int *p, int v, size_t n) {
     const size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
@@ -927,7 +938,8 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
                                                uint32_t seg_stride, int k_eff, int k_floor,
                                                float *__restrict__ out_scores, int64_t *__restrict__ out_idx,
                                                uint32_t *__restrict__ overflow, int *__restrict__ tau_out,
-                                               int tau_stride_q, int keep_floor) {
+                                               int tau_stride_q, int keep_floor, int *__restrict__ raise_out,
+                                               const uint32_t *__restrict__ row_map) {
     __shared__ uint64_t keys[kFinalCap];
     __shared__ uint32_t wave_sum[kFinalThreads / 64];
     __shared__ uint32_t any_full, long_n;
@@ -959,10 +971,17 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
     uint32_t base = incl - mine, total = 0;
     for (int w = 0; w < kFinalThreads / 64; ++w) { if (w < (t >> 6)) base += wave_sum[w]; total += wave_sum[w]; }
     const bool too_many = total > uint32_t(kFinalCap);
+    // A final pass whose candidates did not fit: flag 1 = the caller repeats the full scan for this
+    // query with the raised floor written below (the k_floor-th best of what was kept -- real
+    // slots, so a valid lower bound of the true k-th best, and above the floor that let too many
+    // through); flag 2 = straight to the exact path (no such floor: fewer than k_eff candidates,
+    // or the caller takes no raised floors).
+    bool raising = false;
     if (!sampling) {
         const bool redo = too_many || any_full || total < uint32_t(k_eff);
-        if (t == 0) overflow[qn] = redo ? 1u : 0u;   // set: the caller redoes this query through the exact path
-        if (redo) return;
+        raising = redo && raise_out != nullptr && total >= uint32_t(k_eff);
+        if (t == 0) overflow[qn] = redo ? (raising ? 1u : 2u) : 0u;
+        if (redo && !raising) return;
     }
     if (sampling && total < uint32_t(k_eff)) {
         // Too few allowed slots reached the floor in this sample.  The floor of the level before
@@ -1024,7 +1043,7 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
             if (ok[u]) keys[at[u]] = v[u];
     }
     const uint32_t c_all = min(total, uint32_t(kFinalCap));
-    const uint32_t need = sampling ? min(uint32_t(k_floor), c_all) : uint32_t(k_eff);   // leading keys wanted, in order
+    const uint32_t need = (sampling || raising) ? min(uint32_t(k_floor), c_all) : uint32_t(k_eff);   // leading keys wanted, in order
     uint32_t sort_n = need <= 64u ? 64u : 2u;
     while (sort_n < c_all) sort_n <<= 1;
     __syncthreads();
@@ -1090,21 +1109,22 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
             }
         }
     }
-    if (sampling) {
+    if (sampling || raising) {
         if (t == 0) {
             // the floor: the k_floor-th best sampled score (k_floor >= k_eff steadies the estimate)
             const uint32_t pick = min(uint32_t(k_floor), c_all) - 1;
             float s; uint32_t idx;
             sort_unkey(keys[pick], s, idx);
-            *tau_slot = order_key(s == 0.0f ? -0.0f : s);
+            *(sampling ? tau_slot : raise_out + qn) = order_key(s == 0.0f ? -0.0f : s);
         }
         return;
     }
+    const size_t row = row_map ? size_t(row_map[qn]) : size_t(qn);   // a repeated pass writes to the rows of the queries it repeats
     for (int jj = t; jj < k_eff; jj += kFinalThreads) {
         float s; uint32_t idx;
         sort_unkey(keys[jj], s, idx);
-        out_scores[size_t(qn) * k_eff + jj] = s;
-        out_idx[size_t(qn) * k_eff + jj] = int64_t(idx);
+        out_scores[row * k_eff + jj] = s;
+        out_idx[row * k_eff + jj] = int64_t(idx);
     }
 }
 
@@ -1185,6 +1205,14 @@ hipError_t launch_move_lane(uint8_t *d_native, float *d_scales, const Geometry &
                             hipStream_t s) {
     hipLaunchKernelGGL(k_move_lane, dim3(unsigned((g.G + 255) / 256)), dim3(256), 0, s, d_native, d_scales, g.G,
                        g.nch, src, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_gather_redo(const float *d_q, const uint32_t *d_rows, const int *d_raised, int dim, int tile_q,
+                              size_t n_redo, float *d_q_out, int *d_tau_out, hipStream_t s) {
+    if (n_redo == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_gather_redo, dim3(unsigned(n_redo)), dim3(256), 0, s, d_q, d_rows, d_raised, dim, tile_q,
+                       d_q_out, d_tau_out);
     return hipGetLastError();
 }
 
@@ -1379,10 +1407,11 @@ hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, cons
 
 hipError_t launch_final(const uint64_t *cand, const uint32_t *cand_cnt, uint32_t n_seg, uint32_t seg_stride,
                         int k_eff, int k_floor, int nq, float *out_scores, int64_t *out_idx, uint32_t *overflow,
-                        int *tau_out, int tau_stride_q, int keep_floor, hipStream_t s) {
+                        int *tau_out, int tau_stride_q, int keep_floor, int *raise_out, const uint32_t *row_map,
+                        hipStream_t s) {
     if (nq == 0 || k_eff == 0) return hipSuccess;
     hipLaunchKernelGGL(k_final, dim3(nq), dim3(kFinalThreads), 0, s, cand, cand_cnt, n_seg, seg_stride, k_eff, k_floor,
-                       out_scores, out_idx, overflow, tau_out, tau_stride_q, keep_floor);
+                       out_scores, out_idx, overflow, tau_out, tau_stride_q, keep_floor, raise_out, row_map);
     return hipGetLastError();
 }
 
