@@ -32,7 +32,12 @@ def masks_for(T, n, seed):
                                       (256, 20_011, 333), (384, 9_001, 130), (512, 12_345, 200), (768, 7_003, 290),
                                       (1024, 4_001, 129), (128, 30_011, 400), (640, 5_003, 140), (896, 4_001, 200),
                                       (1152, 3_001, 130), (1408, 3_003, 100), (1792, 2_001, 100), (2304, 2_003, 129),
-                                      (2816, 1_501, 160)])
+                                      (2816, 1_501, 160),
+                                      # row lengths that are not a whole number of chunk pairs: padded with zero
+                                      # chunks to the next instance (1600: 25 -> 26 chunks, 2080: 33 -> 36,
+                                      # 1000 and 200: partly filled last chunk)
+                                      (1600, 3_001, 140), (2080, 2_001, 130), (1000, 4_001, 150), (200, 20_011, 333),
+                                      (1736, 2_501, 129), (2952, 1_203, 131)])
 def test_wide_scan_matches_oracle(T, oracle, dim, n, nq):
     oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=dim + n))
     q = unit_gaussian(nq, dim, seed=77)
@@ -44,6 +49,22 @@ def test_wide_scan_matches_oracle(T, oracle, dim, n, nq):
             os_, oi = oidx.search(q, k, mask_words=words)
             assert np.array_equal(i, oi), k
             assert bits_equal(s, os_), k
+    ix.close()
+
+
+def test_rows_beyond_the_wide_kernel_fall_back_exactly(T, oracle):
+    """More than 48 chunks (over 3072 dimensions at 4 bits): no all-queries-per-pass instance,
+    the tile-group kernels serve the batch, results unchanged."""
+    dim, n, nq = 4096, 1_501, 131
+    oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=9))
+    q = unit_gaussian(nq, dim, seed=10)
+    ix = to_native(T, oidx)
+    for words in masks_for(T, n, 8)[:2]:
+        for k in (1, 10, 100):
+            s, i = ix.search(q, k, mask_words=words)
+            assert ix.queries_per_launch() < nq
+            os_, oi = oidx.search(q, k, mask_words=words)
+            assert np.array_equal(i, oi) and bits_equal(s, os_), k
     ix.close()
 
 

@@ -36,7 +36,7 @@ enum { kModeLists = 0,   // per-lane top-k lists (written out for k_merge)
 struct Geometry {
     int dim = 0, bits = 0;
     int G = 0;    // byte groups per vector = dim*bits/8 (3-bit: dim/2)
-    int nch = 0;  // chunks per block = ceil(G/32)
+    int nch = 0;  // chunks per block: ceil(G/32), plus padding chunks for some 4-bit row lengths (tv_index_create)
     size_t block_bytes() const { return size_t(nch) * 1024; }
 };
 
