@@ -30,6 +30,58 @@ def test_library_exports_every_declared_symbol(T):
         assert hasattr(handle, name), name
 
 
+_C_TO_RUST = {
+    "int": "c_int", "size_t": "usize", "float": "c_float", "double": "c_double", "void": "c_void",
+    "uint8_t": "u8", "uint32_t": "u32", "uint64_t": "u64", "int32_t": "i32", "int64_t": "i64",
+    "tv_index": "tv_index", "char": "c_char",
+}
+
+
+def _rust_type(c_decl):
+    """'const float *queries' -> ('queries', '*const c_float'); 'tv_index **out' -> ('out', '*mut *mut tv_index')."""
+    c_decl = c_decl.strip()
+    m = re.match(r"^(const\s+)?(\w+)\s*(\*{0,2})\s*(\w+)$", c_decl)
+    assert m, c_decl
+    const, base, stars, name = m.groups()
+    t = _C_TO_RUST[base]
+    for depth in range(len(stars)):
+        innermost = depth == 0
+        t = ("*const " if (const and innermost) else "*mut ") + t
+    return name, t
+
+
+def test_rust_bindings_match_the_header():
+    """rust/turbovec-hip-sys/src/lib.rs cannot be compiled here (no Rust toolchain): keep it equal to
+    the C header mechanically -- every entry point, argument names, order and types, return types,
+    and the status / score-mode constants."""
+    header = open(os.path.join(ROOT, "include", "turbovec_hip.h")).read()
+    rust = open(os.path.join(ROOT, "rust", "turbovec-hip-sys", "src", "lib.rs")).read()
+    c_protos = re.findall(r"^(int|size_t|const char \*)\s*(tv_\w+)\s*\(([^;]*?)\)\s*;", header, flags=re.M | re.S)
+    r_protos = {name: (args, ret) for name, args, ret in
+                re.findall(r"pub fn (tv_\w+)\(([^)]*)\)\s*(?:->\s*([^;]+))?;", rust)}
+    assert {p[1] for p in c_protos} == set(r_protos), {p[1] for p in c_protos} ^ set(r_protos)
+    for ret, name, args in c_protos:
+        want_ret = {"int": "c_int", "size_t": "usize", "const char *": "*const c_char"}[ret]
+        assert r_protos[name][1].strip() == want_ret, name
+        c_args = [a for a in (x.strip() for x in " ".join(args.split()).split(",")) if a and a != "void"]
+        r_args = [a.strip() for a in r_protos[name][0].split(",") if a.strip()]
+        assert len(c_args) == len(r_args), name
+        for ca, ra in zip(c_args, r_args):
+            rname, rtype = (x.strip() for x in ra.split(":"))
+            assert (rname, rtype) == _rust_type(ca), (name, ca, ra)
+    for cname, value in re.findall(r"^\s*(TV_[A-Z0-9_]+)\s*=\s*(\d+)", header, flags=re.M):
+        assert re.search(rf"pub const {cname}: c_int = {value};", rust), cname
+
+
+def test_integration_doc_lists_every_binding_entry_point():
+    """INTEGRATION.md names every non-diagnostic entry point of the header."""
+    header = open(os.path.join(ROOT, "include", "turbovec_hip.h")).read()
+    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    declared = set(re.findall(r"\b(tv_[a-z0-9_]+)\s*\(", header)) - {"tv_index"}
+    missing = {n for n in declared if not n.startswith("tv_debug_") and n not in doc}
+    assert not missing, missing
+
+
 def test_status_strings(T):
     L = T.lib()
     assert L.tv_status_string(0) == b"ok"
