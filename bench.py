@@ -34,9 +34,11 @@ sys.path.insert(0, ROOT)
 # HBM bytes one launch of the dominant kernel moves (reads + writes), from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this same command, each scaled by the copy-probe factor (see profiles/).
 MEASURED_TRAFFIC = {
-    ("k_scan_p4_wide", 10_000_000, 1536, 4): 7.7957e9,    # 3,775,883 x 2 KiB fetched + 61,218 KiB written
+    ("k_scan_p4_wide", 10_000_000, 1536, 4): 7.7949e9,    # 3,775,890 x 2 KiB fetched + 60,390 KiB written
     ("k_scan_p4_multi", 10_000_000, 1536, 4): 7.7385e9,   # 3,775,909 x 2 KiB fetched + 5,261 KiB written
-    ("k_scan_p4", 10_000_000, 1536, 4): 7.7206e9,         # 3,769,793 x 2 KiB fetched + 68 KiB written
+    ("k_scan_p4", 10_000_000, 1536, 4): 7.7206e9,         # 3,769,810 x 2 KiB fetched + 56 KiB written
+    ("k_scan_lut_bt", 10_000_000, 1536, 2): 3.8802e9,     # 1,894,650 x 2 KiB fetched
+    ("k_scan_lut", 10_000_000, 1536, 2): 3.8809e9,        # 1,894,970 x 2 KiB fetched
 }
 
 
@@ -149,11 +151,12 @@ def config3_extra(T, torch, build_index, run, args):
     for nq, steps in ((1024, max(3, args.steps // 2)), (1, max(args.steps, 15))):
         dt, scan_ms, launches, q_full = run(nq, steps, 1, ix=ix, k=k, dim=dim)
         launch_s = scan_ms * 1e-3 / max(launches, 1)
+        kern = "k_scan_lut_bt" if q_full == 1 else "k_scan_lut"     # byte tables serve single queries
         res[f"batch{nq}"] = {"queries_per_s": nq * steps / dt, "ms_per_step": dt / steps * 1e3,
                              "queries_per_launch": q_full, "scan_launch_ms": launch_s * 1e3,
                              "roofline": {"bound": "hbm", "achieved": alg / launch_s / 1e9, "peak": 8000.0,
                                           "unit": "GB/s", "frac": alg / launch_s / 1e9 / 8000.0,
-                                          "traffic": None, "kernel": "k_scan_lut"}}
+                                          "traffic": MEASURED_TRAFFIC.get((kern, n, dim, bits)), "kernel": kern}}
     res["overflow_redos"] = ix.overflow_redos()
     ix.close()
     return res
@@ -332,7 +335,7 @@ def main():
     if mode_p:
         kernel = "k_scan_p4_wide" if q_full >= 256 else "k_scan_p4_multi" if q_full > 32 else "k_scan_p4"
     else:
-        kernel = "k_scan_lut"
+        kernel = "k_scan_lut_bt" if q_full == 1 else "k_scan_lut"
     traffic = MEASURED_TRAFFIC.get((kernel, n, dim, bits))
     int8_ops = 2.0 * q_per_launch * n * dim        # multiply-adds x2 of one launch, permute-dot mode
 
