@@ -131,12 +131,18 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
     // a few groups x QL queries), and B[k][n] = 1 where byte k belongs to query n adds them up
     // per query in 32-bit integers while the vector ALU moves on to the next addresses.
     constexpr bool MF = LUT_LDS && (QL == 4 || QL == 8);
+    // 16x16x64: a lane's 16 bytes are row (lane % 16) of k-block (lane / 16).  Lanes 0-15 and 32-47
+    // hold vectors 0-15 (the two halves of a chunk's groups), lanes 16-31 and 48-63 vectors 16-31:
+    // the one-hot B sends the odd k-blocks to a second set of QL output columns, so that one
+    // instruction sums 64 bytes for each of 16 rows and no column is idle at 8 queries.
     v4i bsel = {0, 0, 0, 0};
     {
-        const int n = threadIdx.x & 31;
-        if (QL == 4) { const int w = n < 4 ? int(1u << (8 * n)) : 0; bsel = v4i{w, w, w, w}; }
+        const int n = threadIdx.x & 15, kb = (threadIdx.x >> 4) & 3;
+        const bool mine = n < 2 * QL && (n / QL) == (kb & 1);
+        const int qn = n % QL;
+        if (QL == 4) { const int w = mine ? int(1u << (8 * qn)) : 0; bsel = v4i{w, w, w, w}; }
         if (QL == 8) {
-            const int w0 = n < 4 ? int(1u << (8 * n)) : 0, w1 = (n >= 4 && n < 8) ? int(1u << (8 * (n - 4))) : 0;
+            const int w0 = mine && qn < 4 ? int(1u << (8 * qn)) : 0, w1 = mine && qn >= 4 ? int(1u << (8 * (qn - 4))) : 0;
             bsel = v4i{w0, w1, w0, w1};
         }
     }
@@ -197,7 +203,7 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
         uint32_t acc[QL];
 #pragma unroll
         for (int qq = 0; qq < QL; ++qq) acc[qq] = 0;
-        v16i macc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        v4i macc = {0, 0, 0, 0}, macc2 = {0, 0, 0, 0};   // two chains, so that dependent MFMAs do not queue
         word_t wh[16], wl[16];
         for (int c0 = 0; c0 < nch; c0 += U) {
             uint4 cur[U];
@@ -244,18 +250,21 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
                     constexpr int WPA = 16 / QL;   // words per A operand
 #pragma unroll
                     for (int m = 0; m < 16 / WPA; ++m) {
-                        macc = __builtin_amdgcn_mfma_i32_32x32x32_i8(lut_a_operand<QL>(wh, m), bsel, macc, 0, 0, 0);
-                        macc = __builtin_amdgcn_mfma_i32_32x32x32_i8(lut_a_operand<QL>(wl, m), bsel, macc, 0, 0, 0);
+                        macc = __builtin_amdgcn_mfma_i32_16x16x64_i8(lut_a_operand<QL>(wh, m), bsel, macc, 0, 0, 0);
+                        macc2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(lut_a_operand<QL>(wl, m), bsel, macc2, 0, 0, 0);
                     }
                 }
                 if ((c & 7) == 7 || c == nch - 1) {  // end of a 256-group batch (search.rs:529-531)
                     if (MF) {
-                        // query q's sums sit in the lanes of output column q: hand them to the lanes
-                        // of their vectors through the wave's scratch rows
+                        // lane l holds output column l % 16 (query n % QL of vector half n / QL), rows
+                        // 4 * (l / 16) .. + 3: hand the sums to the lanes of their vectors through the
+                        // wave's scratch rows
                         int *xch = reinterpret_cast<int *>(my_sct);
-                        if (vi < QL) {
+                        const int on = lane & 15;
+                        if (on < 2 * QL) {
 #pragma unroll
-                            for (int r = 0; r < 16; ++r) xch[vi * 32 + 8 * (r >> 2) + 4 * h + (r & 3)] = macc[r];
+                            for (int r = 0; r < 4; ++r)
+                                xch[(on % QL) * 32 + 16 * (on / QL) + 4 * (lane >> 4) + r] = macc[r] + macc2[r];
                         }
                         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
                         __builtin_amdgcn_wave_barrier();
@@ -263,7 +272,8 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
                         for (int qq = 0; qq < QL; ++qq) acc[qq] = uint32_t(xch[qq * 32 + vi]);
                         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
                         __builtin_amdgcn_wave_barrier();
-                        macc = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                        macc = v4i{0, 0, 0, 0};
+                        macc2 = v4i{0, 0, 0, 0};
                     }
 #pragma unroll
                     for (int qq = 0; qq < QL; ++qq) {
