@@ -185,7 +185,8 @@ struct Prepared {
 
 // Query preparation for one chunk: rotation, TQ+ inverse, table build
 // (turbovec/src/search.rs:3237-3269).  d_q holds nq*dim floats on the device.
-int prepare_queries(tv_index *ix, Arena &ar, const float *d_q, size_t nq, Prepared &out) {
+// `split`: permute-dot weights in the order k_scan_p4 reads them (the batched scans take plane order)
+int prepare_queries(tv_index *ix, Arena &ar, const float *d_q, size_t nq, Prepared &out, bool split = true) {
     const tv::Geometry &g = ix->geo;
     const size_t nq_pad = round_up(nq, tv::kQTile);
     const int mode = effective_mode(ix);
@@ -208,7 +209,7 @@ int prepare_queries(tv_index *ix, Arena &ar, const float *d_q, size_t nq, Prepar
         out.table_bytes_per_tile = size_t(g.nch) * 2048;
         out.d_tables = ar.take<uint8_t>(nq_pad / tv::kQTile * out.table_bytes_per_tile);
         TV_HIP(tv::launch_build_p(d_cal, d_bias_corr, out.d_tables, out.d_qscale, out.d_qbias, g.dim, g.G, g.nch,
-                                  ix->cs, nq, nq_pad, ix->stream));
+                                  ix->cs, nq, nq_pad, split, ix->stream));
     } else {
         out.table_bytes_per_tile = size_t(g.nch) * 1024 * tv::kQTile;
         out.d_tables = ar.take<uint8_t>(nq_pad * size_t(g.nch) * 1024);
@@ -499,7 +500,8 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
                 TV_HIP(tv::launch_gather_redo(d_q, d_rows + row0, d_raise, g.dim, int(tile_q), pq_n, d_redo_q, d_tau, ix->stream));
             Prepared pq;
             size_t n_timed = 0;
-            prc = prepare_queries(ix, ar, repeat ? d_redo_q : d_q, pq_n, pq);
+            const int nt_batched = (mode_p && pq_n > size_t(tv::kQTile) && !ix->no_batched) ? tv::batched_tiles(g.nch) : 0;
+            prc = prepare_queries(ix, ar, repeat ? d_redo_q : d_q, pq_n, pq, !wide && nt_batched == 0);
             if (prc != TV_OK) return prc;
             uint64_t *d_cand = ar.take<uint64_t>(cq_pad * seg_stride * tv::kSegCap);
             uint32_t *d_cnt = ar.take<uint32_t>(cq_pad * seg_stride);
@@ -507,7 +509,6 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             // no per-search clears: the first level reads the index's standing array of open floors,
             // every later one the floors k_final wrote, and k_final writes every overflow flag
 
-            const int nt_batched = (mode_p && pq_n > size_t(tv::kQTile) && !ix->no_batched) ? tv::batched_tiles(g.nch) : 0;
             const int bgrid = tv::batched_grid_blocks(ix->device, g.nch);
             for (size_t lv = 0; lv < steps.size(); ++lv) {
                 const bool last = lv + 1 == steps.size();

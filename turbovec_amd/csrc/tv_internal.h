@@ -89,7 +89,7 @@ hipError_t launch_calibrate(const float *d_qrot, float *d_qcal, float *d_bias_co
                             const float *d_scale, int dim, size_t nq, hipStream_t s);
 hipError_t launch_build_p(const float *d_qcal, const float *d_bias_corr, uint8_t *d_wfrag, float *d_qscale,
                           float *d_qbias, int dim, int G, int nch, float cs, size_t nq, size_t nq_padded,
-                          hipStream_t s);
+                          bool split, hipStream_t s);
 hipError_t launch_build_lut(const float *d_qcal, const float *d_bias_corr, const float *d_centroids, uint8_t *d_lut,
                             float *d_qscale, float *d_qbias, int dim, int bits, int G, int nch, size_t nq,
                             size_t nq_padded, hipStream_t s);

@@ -190,15 +190,31 @@ __device__ __forceinline__ float clamp_round_i8(float v) {
 }
 
 // turbovec/src/search.rs:2806-2846 build_permute_dot, emitting the weights in
-// the MFMA B-fragment order of the scan: for query tile t, chunk c and nibble
-// plane p (0 = low nibble = odd dimension, 1 = high nibble = even dimension) a
-// 1 KiB fragment whose lane (h*32 + n) holds the 16 weights of query n for
-// groups 32c + 16h .. +15.
+// the MFMA B-fragment order of the scan.  Plane order (the batched scans, whose
+// decode yields one A operand of low nibbles and one of high nibbles per chunk):
+// for query tile t, chunk c and nibble plane p (0 = low nibble = odd dimension,
+// 1 = high nibble = even dimension) a 1 KiB fragment whose lane (h*32 + n) holds
+// the 16 weights of query n for groups 32c + 16h .. +15.  Split order (k_scan_p4,
+// which decodes the first 8 code bytes of a lane on the vector ALU, four at a
+// time, and looks the other 8 up whole, both levels of a byte side by side):
+// fragment 0 of chunk c holds, in lane (h*32 + n), for e = 0..7, the plane-p
+// weight of group 32c + 16h + e at byte 8*(e/4) + 4p + e%4; fragment 1 the
+// plane-p weight of group 32c + 16h + 8 + e at byte 2e + p.
+__device__ __forceinline__ size_t wfrag_offset(int g, int n, int plane, bool split) {
+    const size_t lane16 = size_t(((g & 31) >> 4) * 32 + n) * 16;
+    if (split) {
+        const int e = g & 7;
+        const int at = (g & 8) ? 2 * e + plane : 8 * (e >> 2) + 4 * plane + (e & 3);
+        return size_t(g >> 5) * 2048 + size_t((g & 15) >> 3) * 1024 + lane16 + size_t(at);
+    }
+    return size_t(g >> 5) * 2048 + size_t(plane) * 1024 + lane16 + size_t(g & 15);
+}
+
 __global__ __launch_bounds__(256) void k_build_p(const float *__restrict__ qcal,
                                                  const float *__restrict__ bias_corr,
                                                  uint8_t *__restrict__ wfrag, float *__restrict__ qscale,
                                                  float *__restrict__ qbias, int dim, int G, int nch, float cs,
-                                                 size_t nq) {
+                                                 size_t nq, bool split) {
     __shared__ float red[4];
     const size_t qi = blockIdx.x;
     const size_t tile = qi / kQTile;
@@ -207,9 +223,8 @@ __global__ __launch_bounds__(256) void k_build_p(const float *__restrict__ qcal,
     const int t = threadIdx.x;
     if (qi >= nq) {  // padding query of the last tile: zero weights
         for (int g = t; g < nch * 32; g += 256) {
-            const size_t off = size_t(g >> 5) * 2048 + size_t(((g & 31) >> 4) * 32 + n) * 16 + size_t(g & 15);
-            base[off] = 0;
-            base[off + 1024] = 0;
+            base[wfrag_offset(g, n, 0, split)] = 0;
+            base[wfrag_offset(g, n, 1, split)] = 0;
         }
         if (t == 0) { qscale[qi] = 0.0f; qbias[qi] = 0.0f; }
         return;
@@ -226,9 +241,8 @@ __global__ __launch_bounds__(256) void k_build_p(const float *__restrict__ qcal,
             lo = int8_t(clamp_round_i8(q[2 * g + 1] * inv_qs));
             hi = int8_t(clamp_round_i8(q[2 * g] * inv_qs));
         }
-        const size_t off = size_t(g >> 5) * 2048 + size_t(((g & 31) >> 4) * 32 + n) * 16 + size_t(g & 15);
-        base[off] = uint8_t(lo);
-        base[off + 1024] = uint8_t(hi);
+        base[wfrag_offset(g, n, 0, split)] = uint8_t(lo);
+        base[wfrag_offset(g, n, 1, split)] = uint8_t(hi);
     }
     if (t == 0) {
         qscale[qi] = cs * qs;
@@ -320,15 +334,52 @@ __global__ __launch_bounds__(256) void k_build_lut(const float *__restrict__ qca
 // int8 query weights (turbovec/src/search.rs:1392-1567 computes the same
 // integers with vpdpbusd).  acc = sum_d w[d] * level[code[d]], exact in i32;
 // score = fma(f32(acc), scale, bias) * vec_scale (search.rs:1519-1524).
+//
+// k_scan_p4 decodes half of a chunk through LDS: a 256-entry table maps a code
+// byte to the two levels of its nibbles (low nibble's in the low byte); two
+// entries make one dword of an A operand -- one shift (the byte's table
+// offset), one LDS read and half a merge per code byte, against 3.75
+// vector-ALU instructions per byte for the in-register lookup, which alone held
+// this kernel below the HBM stream (as does one LDS instruction per byte alone).
+// The table sits at the start of the kernel's LDS (there is no static
+// allocation before it), so a byte's offset is its address.
 // ===========================================================================
+constexpr int kDecodeBytes = 512;
+
+// A 16-bit LDS load, zero-extended, requested without telling the compiler's wait-count
+// bookkeeping (lds_settle is the matching wait).  The loads that fill one half of a register
+// and keep the other are no use here: with ECC-protected register files they clear it.
+__device__ __forceinline__ void lds_u16(uint32_t &dst, uint32_t addr) {
+    asm volatile("ds_read_u16 %0, %1" : "=v"(dst) : "v"(addr));
+}
+// 2 * byte E of x: the offset of that code byte's table entry.
+template <int E>
+__device__ __forceinline__ uint32_t byte_x2(uint32_t x) {
+    uint32_t r;
+    if (E == 0) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0" : "=v"(r) : "v"(1u), "v"(x));
+    if (E == 1) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1" : "=v"(r) : "v"(1u), "v"(x));
+    if (E == 2) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2" : "=v"(r) : "v"(1u), "v"(x));
+    if (E == 3) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3" : "=v"(r) : "v"(1u), "v"(x));
+    return r;
+}
+// 16 bytes of LDS per lane, requested the same way.
+template <int OFF>
+__device__ __forceinline__ void lds_b128(v4i &dst, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(dst) : "v"(addr), "n"(OFF));
+}
+// Hold until at most N LDS requests younger than those feeding e, o, w0 and w1 are outstanding.
+template <int N>
+__device__ __forceinline__ void lds_settle(uint32_t (&e)[4], uint32_t (&o)[4], v4i &w0, v4i &w1) {
+    asm volatile("s_waitcnt lgkmcnt(%10)" : "+v"(e[0]), "+v"(e[1]), "+v"(e[2]), "+v"(e[3]), "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]), "+v"(w0), "+v"(w1) : "n"(N));
+}
 
 template <int U, int MODE, bool W_LDS>
 __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr bool LISTS = MODE == kModeLists, DUMP = MODE == kModeDump, APPEND = MODE == kModeAppend;
     const int nch = a.nch, k = a.k;
-    uint8_t *sW = smem;
-    const size_t w_bytes = W_LDS ? size_t(nch) * 2048 : 0;
+    uint8_t *sW = smem + kDecodeBytes;
+    const size_t w_bytes = kDecodeBytes + (W_LDS ? size_t(nch) * 2048 : 0);
     float *ls = reinterpret_cast<float *>(smem + w_bytes);
     uint32_t *li = reinterpret_cast<uint32_t *>(ls + (LISTS ? k * kScanThreads : 0));
     int *stau = reinterpret_cast<int *>(li + (LISTS ? k * kScanThreads : 0));
@@ -339,6 +390,11 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
         const uint4 *src = reinterpret_cast<const uint4 *>(a.tables);
         uint4 *dst = reinterpret_cast<uint4 *>(sW);
         for (int i = tid; i < nch * 128; i += kScanThreads) dst[i] = src[i];
+    }
+    for (int b = tid; b < 256; b += kScanThreads) {
+        const uint32_t lo = (a.lv[(b & 15) >> 2] >> (8 * (b & 3))) & 0xffu;
+        const uint32_t hi = (a.lv[b >> 6] >> (8 * ((b >> 4) & 3))) & 0xffu;
+        reinterpret_cast<uint16_t *>(smem)[b] = uint16_t(lo | (hi << 8));
     }
     if (LISTS && tid < kQTile) stau[tid] = a.gtau[tid];
     if (APPEND && tid < kQTile) scnt[tid] = 0u;
@@ -403,24 +459,51 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
 #pragma unroll
                 for (int u = 0; u < U; ++u) buf[u] = load_stream16(&codes[(size_t(nj_live) * step * nch + u) * 64]);
             }
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int c = c0 + u;
-                const uint32_t x[4] = {cur[u].x, cur[u].y, cur[u].z, cur[u].w};
-                v4i alo, ahi;
-#pragma unroll
-                for (int d = 0; d < 4; ++d) {
-                    alo[d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
-                    ahi[d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
+            // A chunk gives two A operands.  The first, from code bytes 0..7 of the lane, is decoded
+            // on the vector ALU: dwords (low-nibble levels of bytes 0..3, high-nibble levels of bytes
+            // 0..3, the same for bytes 4..7).  The second, from bytes 8..15, through the byte table:
+            // dword r from bytes 8+2r (low half) and 9+2r (high half), each as its (low nibble, high
+            // nibble) pair of levels.  Either unit alone is slower than the HBM stream (3.75 ALU
+            // instructions per byte; one LDS instruction per byte); half each fits under it.  The
+            // LDS requests of chunk u+1 are issued before chunk u is waited for.
+            uint32_t e[2][4], o[2][4];
+            v4i bw0[2], bw1[2];
+            const uint32_t w_addr = uint32_t(kDecodeBytes + c0 * 2048 + lane * 16);
+            auto request = [&](auto uc) {
+                constexpr int u = decltype(uc)::value, p = u & 1;
+                if (W_LDS) {
+                    lds_b128<u * 2048>(bw0[p], w_addr);
+                } else {
+                    const uint4 w = wglob[(size_t(c0 + u) * 2) * 64];
+                    bw0[p] = v4i{int(w.x), int(w.y), int(w.z), int(w.w)};
                 }
-                uint4 wl, wh;
-                if (W_LDS) { wl = wlds[(c * 2) * 64]; wh = wlds[(c * 2 + 1) * 64]; }
-                else { wl = wglob[(size_t(c) * 2) * 64]; wh = wglob[(size_t(c) * 2 + 1) * 64]; }
-                const v4i blo = {int(wl.x), int(wl.y), int(wl.z), int(wl.w)};
-                const v4i bhi = {int(wh.x), int(wh.y), int(wh.z), int(wh.w)};
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo, blo, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi, bhi, acc, 0, 0, 0);
-            }
+                const uint32_t xa = cur[u].z, xb = cur[u].w;
+                lds_u16(e[p][0], byte_x2<0>(xa)); lds_u16(o[p][0], byte_x2<1>(xa));
+                lds_u16(e[p][1], byte_x2<2>(xa)); lds_u16(o[p][1], byte_x2<3>(xa));
+                lds_u16(e[p][2], byte_x2<0>(xb)); lds_u16(o[p][2], byte_x2<1>(xb));
+                lds_u16(e[p][3], byte_x2<2>(xb)); lds_u16(o[p][3], byte_x2<3>(xb));
+                if (W_LDS) {
+                    lds_b128<u * 2048 + 1024>(bw1[p], w_addr);
+                } else {
+                    const uint4 w = wglob[(size_t(c0 + u) * 2 + 1) * 64];
+                    bw1[p] = v4i{int(w.x), int(w.y), int(w.z), int(w.w)};
+                }
+            };
+            request(IntC<0>{});
+            static_for<U>([&](auto uc) {
+                constexpr int u = decltype(uc)::value, p = u & 1;
+                if constexpr (u + 1 < U) request(IntC<u + 1>{});
+                const v4i a0 = {int(levels_of(cur[u].x & 0x0f0f0f0fu, t0, t1, t2, t3)),
+                                int(levels_of((cur[u].x >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3)),
+                                int(levels_of(cur[u].y & 0x0f0f0f0fu, t0, t1, t2, t3)),
+                                int(levels_of((cur[u].y >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3))};
+                if constexpr (u + 1 < U) lds_settle<W_LDS ? 10 : 8>(e[p], o[p], bw0[p], bw1[p]);
+                else lds_settle<0>(e[p], o[p], bw0[p], bw1[p]);
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, bw0[p], acc, 0, 0, 0);
+                const v4i a1 = {int(e[p][0] | (o[p][0] << 16)), int(e[p][1] | (o[p][1] << 16)),
+                                int(e[p][2] | (o[p][2] << 16)), int(e[p][3] | (o[p][3] << 16))};
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, bw1[p], acc, 0, 0, 0);
+            });
         }
 
         // ---- epilogue: lane owns query qn and rows 8*(r/4) + 4*h + r%4 ----
@@ -1250,10 +1333,10 @@ hipError_t launch_calibrate(const float *d_qrot, float *d_qcal, float *d_bias_co
 
 hipError_t launch_build_p(const float *d_qcal, const float *d_bias_corr, uint8_t *d_wfrag, float *d_qscale,
                           float *d_qbias, int dim, int G, int nch, float cs, size_t nq, size_t nq_padded,
-                          hipStream_t s) {
+                          bool split, hipStream_t s) {
     if (nq_padded == 0) return hipSuccess;
     hipLaunchKernelGGL(k_build_p, dim3(unsigned(nq_padded)), dim3(256), 0, s, d_qcal, d_bias_corr, d_wfrag, d_qscale,
-                       d_qbias, dim, G, nch, cs, nq);
+                       d_qbias, dim, G, nch, cs, nq, split);
     return hipGetLastError();
 }
 
@@ -1278,7 +1361,7 @@ hipError_t launch_build_lut(const float *d_qcal, const float *d_bias_corr, const
 static constexpr size_t kLdsBudget = 160 * 1024;
 
 size_t scan_lds_bytes(int mode_p, int nch, int k, int lut_queries) {
-    const size_t lists = size_t(k) * kScanThreads * 8 + kQTile * sizeof(int);
+    const size_t lists = size_t(k) * kScanThreads * 8 + kQTile * sizeof(int) + (mode_p ? kDecodeBytes : 0);
     if (mode_p) {
         const size_t w = size_t(nch) * 2048;
         return (w + lists <= kLdsBudget ? w : 0) + lists;
@@ -1300,7 +1383,7 @@ int scan_grid_blocks(int device, int mode_p, int nch, int k, int nq_tile) {
 
 hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s) {
     const size_t w = size_t(a.nch) * 2048;
-    const size_t lists = mode != kModeLists ? 64 : size_t(a.k) * kScanThreads * 8 + kQTile * sizeof(int);
+    const size_t lists = kDecodeBytes + (mode != kModeLists ? 64 : size_t(a.k) * kScanThreads * 8 + kQTile * sizeof(int));
     const bool w_lds = w + lists <= kLdsBudget;
     const size_t lds = (w_lds ? w : 0) + lists;
     hipError_t e = hipSuccess;
