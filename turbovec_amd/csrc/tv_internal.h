@@ -108,6 +108,7 @@ hipError_t launch_scan_lut(const ScanArgs &a, int grid, int mode, hipStream_t s)
 int batched_tiles(int nch);
 int batched_grid_blocks(int device, int nch);
 hipError_t launch_scan_p4_batched(const ScanArgs &a, int grid, hipStream_t s);
+bool batched_weights_split(int nch);   // which weight order launch_scan_p4_batched's kernel reads
 // out_tau == nullptr: write the k_eff best of the merged lists; else write only the
 // order key of the k_eff-th best (a floor at least k_eff scanned slots reach) per query.
 // Wide batched scan (every query of a chunk in one pass; tv_kernels3.hip).

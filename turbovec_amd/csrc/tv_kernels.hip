@@ -373,6 +373,17 @@ __device__ __forceinline__ void lds_settle(uint32_t (&e)[4], uint32_t (&o)[4], v
     asm volatile("s_waitcnt lgkmcnt(%10)" : "+v"(e[0]), "+v"(e[1]), "+v"(e[2]), "+v"(e[3]), "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]), "+v"(w0), "+v"(w1) : "n"(N));
 }
 
+// The same with a run-time address, and a full wait tied to the registers a step is about to use.
+__device__ __forceinline__ void lds_b128_at(v4i &dst, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1" : "=&v"(dst) : "v"(addr));
+}
+template <int NT>
+__device__ __forceinline__ void lds_settle_all(uint32_t (&e)[4], uint32_t (&o)[4], v4i (&w)[NT]) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e[0]), "+v"(e[1]), "+v"(e[2]), "+v"(e[3]), "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
+#pragma unroll
+    for (int t = 0; t < NT; ++t) asm volatile("" : "+v"(w[t]));
+}
+
 template <int U, int MODE, bool W_LDS>
 __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
@@ -591,8 +602,8 @@ template <int NT, int U, int THREADS>
 __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     const int nch = a.nch;
-    uint8_t *sW = smem;                                            // [NT][nch][2][64 lanes][16]
-    uint32_t *scnt = reinterpret_cast<uint32_t *>(smem + size_t(NT) * nch * 2048);
+    uint8_t *sW = smem + kDecodeBytes;                             // [NT][nch][2][64 lanes][16], after the byte table
+    uint32_t *scnt = reinterpret_cast<uint32_t *>(sW + size_t(NT) * nch * 2048);
     const int tid = threadIdx.x, lane = tid & 63;
     const int qn = lane & 31, h = lane >> 5;
     const int nt_active = (a.nq_tile + kQTile - 1) / kQTile;
@@ -601,6 +612,11 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
         uint4 *dst = reinterpret_cast<uint4 *>(sW);
         const int live16 = nt_active * nch * 128;
         for (int i = tid; i < NT * nch * 128; i += THREADS) dst[i] = i < live16 ? src[i] : make_uint4(0, 0, 0, 0);
+    }
+    for (int b = tid; b < 256; b += THREADS) {   // code byte -> (level of its low nibble, level of its high nibble)
+        const uint32_t lo = (a.lv[(b & 15) >> 2] >> (8 * (b & 3))) & 0xffu;
+        const uint32_t hi = (a.lv[b >> 6] >> (8 * ((b >> 4) & 3))) & 0xffu;
+        reinterpret_cast<uint16_t *>(smem)[b] = uint16_t(lo | (hi << 8));
     }
     for (int i = tid; i < NT * kQTile; i += THREADS) scnt[i] = 0u;
     uint32_t *snext = scnt + NT * kQTile;   // next unclaimed block of this workgroup
@@ -625,7 +641,7 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
     const uint32_t step = a.b_step;
     const uint32_t nj = (a.n_blocks + step - 1) / step;
     const uint4 *codes = reinterpret_cast<const uint4 *>(a.codes) + lane;
-    const uint4 *wlds = reinterpret_cast<const uint4 *>(sW) + lane;
+    const uint32_t w_base = uint32_t(kDecodeBytes + lane * 16), w_tile = uint32_t(nch) * 2048u;
 
     // Blocks are dealt round-robin to workgroups (logical block m * gridDim.x + blockIdx.x belongs
     // to this one), so neighbouring rows -- clustered data, contiguous allowlists -- spread over
@@ -711,25 +727,37 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
             if (u == 1) wait_vm<2 * U - 1>(cur[U > 1 ? 1 : 0]);
             if (u == 2) wait_vm<2 * U - 2>(cur[U > 2 ? 2 : 0]);
             if (u == 3) wait_vm<2 * U - 3>(cur[U > 3 ? 3 : 0]);
-            const uint32_t x[4] = {cur[u].x, cur[u].y, cur[u].z, cur[u].w};
-            v4i alo, ahi;
+            // Split decode as in k_scan_p4: code bytes 8..15 of the lane through the byte table
+            // (requested first), bytes 0..7 on the vector ALU while those reads and the first
+            // operand's weights are on their way; the second operand's weights travel during the
+            // first operand's MFMAs.  All LDS traffic of the loop is requested and waited for by
+            // hand, so the counts below are exact.
+            uint32_t e[4], o[4];
+            lds_u16(e[0], byte_x2<0>(cur[u].z)); lds_u16(o[0], byte_x2<1>(cur[u].z));
+            lds_u16(e[1], byte_x2<2>(cur[u].z)); lds_u16(o[1], byte_x2<3>(cur[u].z));
+            lds_u16(e[2], byte_x2<0>(cur[u].w)); lds_u16(o[2], byte_x2<1>(cur[u].w));
+            lds_u16(e[3], byte_x2<2>(cur[u].w)); lds_u16(o[3], byte_x2<3>(cur[u].w));
+            const uint32_t w_addr = w_base + uint32_t(c) * 2048u;
+            v4i b0[NT], b1[NT];
+            static_for<NT>([&](auto tc) {
+                constexpr int t = decltype(tc)::value;
+                lds_b128_at(b0[t], w_addr + uint32_t(t) * w_tile);
+            });
+            const v4i a0 = {int(levels_of(cur[u].x & 0x0f0f0f0fu, t0, t1, t2, t3)),
+                            int(levels_of((cur[u].x >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3)),
+                            int(levels_of(cur[u].y & 0x0f0f0f0fu, t0, t1, t2, t3)),
+                            int(levels_of((cur[u].y >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3))};
+            lds_settle_all(e, o, b0);
+            static_for<NT>([&](auto tc) {
+                constexpr int t = decltype(tc)::value;
+                lds_b128_at(b1[t], w_addr + uint32_t(t) * w_tile + 1024u);
+            });
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                alo[d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
-                ahi[d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
-            }
+            for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b0[t], acc[t], 0, 0, 0);
+            const v4i a1 = {int(e[0] | (o[0] << 16)), int(e[1] | (o[1] << 16)), int(e[2] | (o[2] << 16)), int(e[3] | (o[3] << 16))};
+            lds_settle_all(e, o, b1);
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                const uint4 wl = wlds[(size_t(t) * nch + c) * 128];
-                const v4i blo = {int(wl.x), int(wl.y), int(wl.z), int(wl.w)};
-                acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo, blo, acc[t], 0, 0, 0);
-            }
-#pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                const uint4 wh = wlds[(size_t(t) * nch + c) * 128 + 64];
-                const v4i bhi = {int(wh.x), int(wh.y), int(wh.z), int(wh.w)};
-                acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi, bhi, acc[t], 0, 0, 0);
-            }
+            for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b1[t], acc[t], 0, 0, 0);
         }
         if (block_ends) {
             wait_vm<U + 1>(cur_sc);   // this group's own scale: only the request issued above is younger
@@ -1416,12 +1444,15 @@ hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s) 
 // Query tiles whose weights fit LDS together, capped at 4.
 static int resident_tiles(int nch) {
     const size_t per_tile = size_t(nch) * 2048;
-    int nt = int((kLdsBudget - 1024) / per_tile);
+    int nt = int((kLdsBudget - 1024 - kDecodeBytes) / per_tile);
     return nt > 4 ? 4 : nt;
 }
 
 constexpr int kMultiThreads = 768;   // 3 waves per SIMD: measured best of 512 / 768 / 1024
 constexpr int kStreamTiles = 4, kStreamBlocksPerWave = 2, kStreamSliceChunks = 2, kStreamOccupancy = 2;
+
+// The resident-weights kernel reads its weights in k_scan_p4's split order.
+bool batched_weights_split(int nch) { return resident_tiles(nch) >= 2; }
 
 int batched_tiles(int nch) {
     const int nt = resident_tiles(nch);
@@ -1435,7 +1466,7 @@ int batched_grid_blocks(int device, int nch) {
     if (hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0)
         cus = prop.multiProcessorCount;
     if (resident_tiles(nch) >= 2) {
-        const size_t lds = size_t(resident_tiles(nch)) * nch * 2048 + 1024;
+        const size_t lds = size_t(resident_tiles(nch)) * nch * 2048 + 1024 + kDecodeBytes;
         const int per_cu = int(kLdsBudget / lds);
         return cus * (per_cu < 1 ? 1 : (per_cu > 2 ? 2 : per_cu));
     }
@@ -1444,7 +1475,7 @@ int batched_grid_blocks(int device, int nch) {
 
 template <int NT, int U>
 static hipError_t launch_multi_u(const ScanArgs &a, int grid, hipStream_t s) {
-    const size_t lds = size_t(NT) * a.nch * 2048 + (NT * kQTile + 1) * sizeof(uint32_t);
+    const size_t lds = kDecodeBytes + size_t(NT) * a.nch * 2048 + (NT * kQTile + 1) * sizeof(uint32_t);
     hipError_t e = allow_lds(k_scan_p4_multi<NT, U, kMultiThreads>, lds);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((k_scan_p4_multi<NT, U, kMultiThreads>), dim3(grid), dim3(kMultiThreads), lds, s, a);
