@@ -37,7 +37,10 @@ def masks_for(T, n, seed):
                                       # chunks to the next instance (1600: 25 -> 26 chunks, 2080: 33 -> 36,
                                       # 1000 and 200: partly filled last chunk)
                                       (1600, 3_001, 140), (2080, 2_001, 130), (1000, 4_001, 150), (200, 20_011, 333),
-                                      (1736, 2_501, 129), (2952, 1_203, 131)])
+                                      (1736, 2_501, 129), (2952, 1_203, 131),
+                                      # rows beyond one wave's registers (over 48 chunks): split over wave pairs
+                                      (4096, 1_501, 131), (3584, 1_203, 260), (4104, 1_001, 129), (5000, 1_003, 150),
+                                      (6144, 1_001, 140), (3200, 1_501, 1029)])
 def test_wide_scan_matches_oracle(T, oracle, dim, n, nq):
     oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=dim + n))
     q = unit_gaussian(nq, dim, seed=77)
@@ -53,9 +56,9 @@ def test_wide_scan_matches_oracle(T, oracle, dim, n, nq):
 
 
 def test_rows_beyond_the_wide_kernel_fall_back_exactly(T, oracle):
-    """More than 48 chunks (over 3072 dimensions at 4 bits): no all-queries-per-pass instance,
+    """More than 96 chunks (over 6144 dimensions at 4 bits): no all-queries-per-pass instance,
     the tile-group kernels serve the batch, results unchanged."""
-    dim, n, nq = 4096, 1_501, 131
+    dim, n, nq = 6400, 1_001, 131
     oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=9))
     q = unit_gaussian(nq, dim, seed=10)
     ix = to_native(T, oidx)

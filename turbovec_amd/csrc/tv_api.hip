@@ -670,9 +670,11 @@ int tv_index_create(int dim, int bits, int device, tv_index **out) {
     ix->geo.nch = (ix->geo.G + tv::kChunkGroups - 1) / tv::kChunkGroups;
     // 4-bit rows are padded with whole chunks of zero groups (their query weights are zero, so they
     // add nothing) up to a chunk count the all-queries-per-pass kernel has an instance for: even
-    // from 9 chunks on, a multiple of 4 above 24.  At most one chunk in nine of extra code bytes.
+    // from 9 chunks on, a multiple of 4 above 24, of 8 above 48 (to 96 chunks = 6144 dimensions).
+    // At most one chunk in nine of extra code bytes.
     if (bits == 4 && ix->geo.nch >= 9) {
-        if (ix->geo.nch > 24 && ix->geo.nch <= 48) ix->geo.nch = (ix->geo.nch + 3) / 4 * 4;
+        if (ix->geo.nch > 48 && ix->geo.nch <= 96) ix->geo.nch = (ix->geo.nch + 7) / 8 * 8;
+        else if (ix->geo.nch > 24 && ix->geo.nch <= 48) ix->geo.nch = (ix->geo.nch + 3) / 4 * 4;
         else if (ix->geo.nch <= 24) ix->geo.nch += ix->geo.nch & 1;
     }
     ix->rot = tv::make_rotation_tables(dim);

@@ -97,17 +97,28 @@ struct WideQuery {
 // NCH / SPT chunks, handed over one by one (HO = 1) or HO at a time.  Short rows leave registers
 // for BLK blocks per wave: every B operand read from LDS then feeds BLK MFMAs, and a tile's
 // barriers and epilogue are shared by BLK times the work.
-template <int NCH, int NB, int WAVES, int SPT, int BLK, int HO>
+//
+// KS = 2 splits a row of 2 * NCH chunks over a pair of waves (w, w + 1): each holds the block's
+// operands for half the row (NCH chunks: what one wave's registers take), walks its half of every
+// tile's weights -- a ring slot then carries both halves of a slice side by side -- and at the
+// end of a tile the odd wave hands its partial sums to the even one through LDS, which adds them
+// and does the tile's bound test and scoring.  Two blocks per workgroup instead of four, one more
+// barrier per tile: the form for rows beyond what one wave holds.
+template <int NCH, int NB, int WAVES, int SPT, int BLK, int HO, int KS>
 __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide(ScanArgs a) {
     static_assert(NCH % SPT == 0, "a slice is a whole number of chunks");
+    static_assert(KS == 1 || (KS == 2 && WAVES == 4 && BLK == 1 && HO == 1), "row halves go to the wave pairs of the four-wave form");
     static_assert(HO == 1 || (SPT % HO == 0 && kWideRing >= 2 * HO + 1), "slices handed over together must fit the ring twice");
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr int kWideThreads = WAVES * 64, kWideWaves = WAVES;
     constexpr int kSC = NCH / SPT;                          // chunks per slice
     constexpr int kM = 2 * kSC;                             // MFMAs per wave and slice: (low, high) of each chunk
     constexpr int kSlice = kM * 1024;                       // bytes: one 1 KiB B operand per MFMA
-    constexpr int kPieces = kM / kWideWaves;                // direct-to-LDS loads per wave and slice ...
-    constexpr int kExtra = kM % kWideWaves;                 // ... plus one more in the first kExtra waves
+    constexpr int kSlot = KS * kSlice;                      // a ring slot: the slice of every row part
+    constexpr int kLoaders = kWideWaves / KS;               // waves that share the loading of one row part's slice
+    constexpr int kPieces = kM / kLoaders;                  // direct-to-LDS loads per wave and slice ...
+    constexpr int kExtra = kM % kLoaders;                   // ... plus one more in the first kExtra waves
+    static_assert(KS == 1 || kExtra == 0, "the pair form deals a slice's pieces evenly");
     constexpr int kAhead = kWideRing - 1;
     // Four-wave forms (one wave per SIMD, up to 48 chunks = 384 operand registers): chunks from
     // kVecChunks on live in accumulation registers and the MFMAs are written by hand.
@@ -118,15 +129,18 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     const int nt = (nq + kQTile - 1) / kQTile;
     const int nq_pad = nt * kQTile;
     const int n_slices = SPT * nt;                          // per pass over the tiles; the host guarantees >= kAhead
-    WideQuery *sq = reinterpret_cast<WideQuery *>(smem + kWideRing * kSlice);
+    WideQuery *sq = reinterpret_cast<WideQuery *>(smem + kWideRing * kSlot);
     float *s_vs = reinterpret_cast<float *>(sq + nq_pad);   // [waves][BLK][32]: row scales, NaN where not allowed
     uint32_t *snext = reinterpret_cast<uint32_t *>(s_vs + kWideWaves * BLK * 32);
+    v4i *s_xch = reinterpret_cast<v4i *>(snext + 16);       // KS = 2: [pairs][4][64 lanes] partial sums on their way
     const uint32_t lds_b = uint32_t(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)smem));
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int qn = lane & 31, h = lane >> 5;
     const uint32_t lane16 = uint32_t(lane) * 16;
+    const int part = KS == 2 ? (wave & 1) : 0;              // which half of the row this wave holds
+    const int loader = KS == 2 ? (wave >> 1) : wave;        // its rank among the waves loading that part's slices
     for (int q = tid; q < nq_pad; q += kWideThreads) {
         const bool act = q < nq;
         const float qs = act ? a.qscale[q] : 0.0f, qb = act ? a.qbias[q] : 0.0f;
@@ -152,12 +166,20 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     const uint32_t step = a.b_step;
     const uint32_t nj = (a.n_blocks + step - 1) / step;
 
-    // next live block of this workgroup (blocks m * gridDim.x + blockIdx.x), claimed wave by wave
+    // next live block of this workgroup (blocks m * gridDim.x + blockIdx.x), claimed wave by wave;
+    // the two waves of a pair must arrive at the same block without talking: pair p takes the
+    // logical blocks m = p, p + pairs, ...
+    uint32_t pair_m = uint32_t(wave >> 1);
     auto claim = [&]() -> uint32_t {
         for (;;) {
             uint32_t m = 0;
-            if (lane == 0) m = atomicAdd(snext, 1u);
-            m = uint32_t(__builtin_amdgcn_readfirstlane(int(m)));
+            if constexpr (KS == 2) {
+                m = pair_m;
+                pair_m += kWideWaves / 2;
+            } else {
+                if (lane == 0) m = atomicAdd(snext, 1u);
+                m = uint32_t(__builtin_amdgcn_readfirstlane(int(m)));
+            }
             const uint32_t j = m * gridDim.x + blockIdx.x;
             if (j >= nj || a.mask == nullptr) return j;
             const uint32_t b = j * step;
@@ -176,13 +198,17 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     // (waves below kExtra request one piece more).
     int req_slice = 0, req_slot = 0;                        // next stream position to request
     auto request_next = [&]() {
-        const uint8_t *src = a.tables + size_t(req_slice) * kSlice + size_t(wave) * 1024;
-        const uint32_t dst = lds_b + uint32_t(req_slot) * kSlice + uint32_t(wave) * 1024;
+        // KS = 1: the stream is contiguous in memory.  KS = 2: a tile holds the first half of the
+        // row's chunks, then the second; slice s is part s % SPT of each half of tile s / SPT.
+        const uint8_t *src = KS == 1 ? a.tables + size_t(req_slice) * kSlice + size_t(loader) * 1024
+                                     : a.tables + size_t(req_slice / SPT) * (size_t(KS) * NCH * 2048) +
+                                           size_t(part) * (NCH * 2048) + size_t(req_slice % SPT) * kSlice + size_t(loader) * 1024;
+        const uint32_t dst = lds_b + uint32_t(req_slot) * kSlot + uint32_t(part) * kSlice + uint32_t(loader) * 1024;
 #pragma unroll
         for (int p = 0; p < kPieces; ++p)
-            dma16_to_lds(dst + uint32_t(p) * (kWideWaves * 1024), src + size_t(p) * (kWideWaves * 1024), lane16);
+            dma16_to_lds(dst + uint32_t(p) * (kLoaders * 1024), src + size_t(p) * (kLoaders * 1024), lane16);
         if (kExtra != 0 && wave < kExtra)
-            dma16_to_lds(dst + uint32_t(kPieces) * (kWideWaves * 1024), src + size_t(kPieces) * (kWideWaves * 1024), lane16);
+            dma16_to_lds(dst + uint32_t(kPieces) * (kLoaders * 1024), src + size_t(kPieces) * (kLoaders * 1024), lane16);
         req_slice = req_slice + 1 == n_slices ? 0 : req_slice + 1;
         req_slot = req_slot + 1 == kWideRing ? 0 : req_slot + 1;
     };
@@ -226,7 +252,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     static_assert(kM % NB == 0 && NB <= kM / 2, "the operand ring must line up with the slices");
     v4i w[NB];
     auto open_stream = [&]() {
-        const uint32_t baddr = lds_b + uint32_t(use_slot) * kSlice + lane16;
+        const uint32_t baddr = lds_b + uint32_t(use_slot) * kSlot + uint32_t(part) * kSlice + lane16;
         static_for<NB>([&](auto mm) { lds_read16_async<decltype(mm)::value * 1024>(w[decltype(mm)::value], baddr); });
     };
     auto close_stream = [&]() {    // the reads into the slice after the round's last are dropped, once landed
@@ -235,16 +261,16 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     // The kM MFMAs of one slice.  MFMA m takes chunk PART * kSC + m/2 (low nibbles for even m,
     // high for odd) against the 1 KiB of weights at m * 1024; the hand-over of the next slice
     // sits in the middle.
-    auto slice_mfmas = [&](auto part) {
-        constexpr int c0 = decltype(part)::value * kSC;
-        const uint32_t baddr = lds_b + uint32_t(use_slot) * kSlice + lane16;
+    auto slice_mfmas = [&](auto slice_no) {
+        constexpr int c0 = decltype(slice_no)::value * kSC;
+        const uint32_t baddr = lds_b + uint32_t(use_slot) * kSlot + uint32_t(part) * kSlice + lane16;
         use_slot = use_slot + 1 == kWideRing ? 0 : use_slot + 1;
-        const uint32_t naddr = lds_b + uint32_t(use_slot) * kSlice + lane16;
+        const uint32_t naddr = lds_b + uint32_t(use_slot) * kSlot + uint32_t(part) * kSlice + lane16;
         static_for<kM>([&](auto mm) {
             constexpr int m = decltype(mm)::value;
             if constexpr (m == kM / 2) {
                 if constexpr (HO == 1) hand_over(IntC<kAhead - 2>{});
-                else if constexpr (decltype(part)::value % HO == HO - 1) hand_over_group();
+                else if constexpr (decltype(slice_no)::value % HO == HO - 1) hand_over_group();
             }
             lds_wait<NB - 1>(w[m % NB]);
             static_for<BLK>([&](auto kk) {
@@ -252,7 +278,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
                 constexpr int c = c0 + m / 2;
                 if constexpr (kHandMfma) {
                     const v4i &A = (m & 1) == 0 ? alo[k][c] : ahi[k][c];
-                    if constexpr (decltype(part)::value == 0 && m == 0) mfma_i8_first<(c >= kVecChunks)>(acc[k], A, w[m % NB]);
+                    if constexpr (decltype(slice_no)::value == 0 && m == 0) mfma_i8_first<(c >= kVecChunks)>(acc[k], A, w[m % NB]);
                     else mfma_i8_add<(c >= kVecChunks)>(acc[k], A, w[m % NB]);
                 } else if constexpr ((m & 1) == 0) {
                     acc[k] = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo[k][c], w[m % NB], acc[k], 0, 0, 0);
@@ -284,7 +310,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
                 // the whole block in one burst: the previous block's operands are dead by now, so
                 // the raw codes (4 VGPRs per chunk) and the operands decoded from them so far (8 per
                 // chunk) fit the registers the operands alone need at the end
-                const uint8_t *p = a.codes + size_t(b) * NCH * 1024;
+                const uint8_t *p = a.codes + (size_t(b) * KS + size_t(part)) * (NCH * 1024);
                 u32x4 raw[NCH];
                 // with hand-written MFMAs the chunks bound for the accumulation registers come
                 // first: their raw codes leave the vector registers before the others' operands grow
@@ -373,9 +399,28 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
                     if (odd_block[k]) bound[k] = int(0x80000000);
                 });
                 static_for<SPT - 1>([&](auto pp) { slice_mfmas(IntC<decltype(pp)::value + 1>{}); });
-                static_for<BLK>([&](auto kk) {
+                if constexpr (KS == 2) {
+                    // the odd wave's half of the sums crosses to the even one; the slot is free
+                    // again by the time it is written next: a hand-over barrier lies in between
+                    mfma_settle(acc[0]);
+                    v4i *x = s_xch + (wave >> 1) * 256 + lane;
+                    if (part == 1) {
+#pragma unroll
+                        for (int r4 = 0; r4 < 4; ++r4)
+                            x[r4 * 64] = v4i{acc[0][4 * r4], acc[0][4 * r4 + 1], acc[0][4 * r4 + 2], acc[0][4 * r4 + 3]};
+                    }
+                    __syncthreads();
+                    if (part == 0) {
+#pragma unroll
+                        for (int r4 = 0; r4 < 4; ++r4) {
+                            const v4i o = x[r4 * 64];
+                            acc[0][4 * r4] += o[0]; acc[0][4 * r4 + 1] += o[1]; acc[0][4 * r4 + 2] += o[2]; acc[0][4 * r4 + 3] += o[3];
+                        }
+                    }
+                }
+                if (KS == 1 || part == 0) static_for<BLK>([&](auto kk) {
                     constexpr int k = decltype(kk)::value;
-                    if constexpr (kHandMfma) mfma_settle(acc[k]);
+                    if constexpr (kHandMfma && KS == 1) mfma_settle(acc[k]);
                     const v16i &c = acc[k];
                     int m0 = max(max(c[0], c[1]), c[2]), m1 = max(max(c[3], c[4]), c[5]);
                     int m2 = max(max(c[6], c[7]), c[8]), m3 = max(max(c[9], c[10]), c[11]);
@@ -392,6 +437,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
 #pragma unroll
                     for (int i = 0; i < SPT / HO; ++i) hand_over_group();
                 }
+                if constexpr (KS == 2) __syncthreads();     // the tile's exchange barrier, met by every wave
             }
         }
         if (has) close_stream();
@@ -464,13 +510,15 @@ int wide_min_queries(int nch) {
         case 2: case 4: case 6: case 8: case 10: case 12: case 14: case 16: case 18: return 129;
         case 20: case 22: case 24: return 97;
         case 28: case 32: case 36: case 40: case 44: case 48: return 97;
+        case 56: case 64: case 72: case 80: case 88: case 96: return 129;
         default: return 0;
     }
 }
 
-static size_t wide_lds_bytes(int slice_bytes, int nq, int blk) {
+static size_t wide_lds_bytes(int slot_bytes, int nq, int blk, int ks) {
     const size_t nq_pad = size_t((nq + kQTile - 1) / kQTile) * kQTile;
-    return size_t(kWideRing) * slice_bytes + nq_pad * sizeof(WideQuery) + size_t(kWideWaves) * blk * 32 * 4 + 64;
+    return size_t(kWideRing) * slot_bytes + nq_pad * sizeof(WideQuery) + size_t(kWideWaves) * blk * 32 * 4 + 64 +
+           (ks == 2 ? 2 * 4096 : 0);
 }
 
 int wide_grid_blocks(int device) {
@@ -481,15 +529,16 @@ int wide_grid_blocks(int device) {
     return cus;      // one 8-wave workgroup per CU: its LDS holds the slice ring
 }
 
-template <int NCH, int NB, int WAVES = 8, int SPT = 2, int BLK = 1, int HO = 1>
+template <int NCH, int NB, int WAVES = 8, int SPT = 2, int BLK = 1, int HO = 1, int KS = 1>
 static hipError_t launch_wide_n(const ScanArgs &a, int grid, hipStream_t s) {
-    const size_t lds = wide_lds_bytes(2 * (NCH / SPT) * 1024, a.nq_tile, BLK);
+    const size_t lds = wide_lds_bytes(KS * 2 * (NCH / SPT) * 1024, a.nq_tile, BLK, KS);
+    if (lds > 160 * 1024) return hipErrorInvalidValue;
     if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK, HO>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK, HO, KS>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK, HO>), dim3(grid), dim3(WAVES * 64), lds, s, a);
+    hipLaunchKernelGGL((k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK, HO, KS>), dim3(grid), dim3(WAVES * 64), lds, s, a);
     return hipGetLastError();
 }
 
@@ -518,6 +567,13 @@ hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s) {
         case 40: return launch_wide_n<40, 4, 4, 4, 1>(a, grid, s);
         case 44: return launch_wide_n<44, 2, 4, 4, 1>(a, grid, s);
         case 48: return launch_wide_n<48, 4, 4, 4, 1>(a, grid, s);
+        // rows beyond one wave's registers, split over wave pairs: <chunks per wave, ..., slices of 4 chunks>
+        case 56: return launch_wide_n<28, 2, 4, 7, 1, 1, 2>(a, grid, s);
+        case 64: return launch_wide_n<32, 2, 4, 8, 1, 1, 2>(a, grid, s);
+        case 72: return launch_wide_n<36, 2, 4, 9, 1, 1, 2>(a, grid, s);
+        case 80: return launch_wide_n<40, 2, 4, 10, 1, 1, 2>(a, grid, s);
+        case 88: return launch_wide_n<44, 2, 4, 11, 1, 1, 2>(a, grid, s);
+        case 96: return launch_wide_n<48, 2, 4, 12, 1, 1, 2>(a, grid, s);
         default: return hipErrorInvalidValue;
     }
 }
