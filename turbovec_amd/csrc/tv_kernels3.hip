@@ -159,7 +159,8 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
         sq[q].ta = !act ? inf : bounded ? (tau / qs) * (1.0f - 1e-5f) : -inf;
         sq[q].tb = act && bounded ? rb + 1e-5f * fabsf(rb) + 2.0f : 0.0f;
     }
-    if (tid == 0) *snext = 0u;
+    if (tid == 0) { snext[0] = 0u; snext[1] = 0u; }
+    uint32_t *s_over = snext + 1;                           // queries whose segment of this workgroup is full
     __syncthreads();
 
     const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
@@ -297,9 +298,15 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     for (;;) {
         // ---- block phase: claim, load, decode into registers ----
         bool has = false;
+        // Once every query's segment of this workgroup is full, every query of the launch is
+        // certain to be flagged as overflowed and scanned again from a raised floor: nothing this
+        // workgroup could still append would be kept, so it claims no further blocks.  (A floor
+        // far too low -- rows arranged against the sampler -- ends the launch within a few rounds
+        // instead of scoring the whole index for nothing.)
+        const bool futile = uint32_t(__builtin_amdgcn_readfirstlane(int(*reinterpret_cast<volatile uint32_t *>(s_over)))) >= uint32_t(nq);
         static_for<BLK>([&](auto kk) {
             constexpr int k = decltype(kk)::value;
-            const uint32_t j = claim();
+            const uint32_t j = futile ? nj : claim();
             const bool has_k = j < nj;
             has = has || has_k;
             const uint32_t b = has_k ? j * step : 0u;
@@ -378,6 +385,8 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
                         if (pos < kSegCap)
                             a.cand[(size_t(q) * a.seg_stride + blockIdx.x) * kSegCap + pos] =
                                 sort_key(s, blk[k] * 32u + uint32_t(i + 4 * h));
+                        else if (pos == kSegCap)
+                            atomicAdd(s_over, 1u);      // the one append that finds the segment just full
                     }
                 }
             }
