@@ -114,6 +114,41 @@ def test_wide_scan_matches_other_paths(T, dim, n, nq):
     ix.close()
 
 
+def test_wide_scan_stops_early_when_every_query_overflows(T):
+    """Rows laid out against the sampler for a whole batch: the one sampling level reads every
+    256th block (8192 blocks, k=10: 1024 sampled slots), those blocks hold the opposite of what
+    the queries look for and every other block near-duplicates of it.  Every query's candidate
+    segments fill within a round, the workgroups of the all-queries-per-pass kernel stop claiming
+    blocks, and the batch is scanned again from raised floors: the answer equals the exact path's
+    and the tile-group kernels', and no query needs the exact path."""
+    dev = torch.device("cuda:0")
+    dim, n, nq = 256, 8192 * 32, 200
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(5)
+    c = torch.randn(dim, device=dev, generator=gen)
+    c = c / c.norm()
+    ix = T.NativeIndex(dim, 4)
+    for c0 in range(0, n, 65_536):
+        m = min(65_536, n - c0)
+        block = (torch.arange(c0, c0 + m, device=dev) // 32)
+        sign = torch.where(block % 256 == 0, -1.0, 1.0).unsqueeze(1)
+        v = sign * c + 0.3 * torch.randn(m, dim, device=dev, generator=gen) / dim ** 0.5
+        torch.cuda.synchronize()
+        ix.add_dev(v.data_ptr(), m)
+    q = (c + 0.3 * torch.randn(nq, dim, device=dev, generator=gen) / dim ** 0.5).cpu().numpy()
+    s, i = ix.search(q, 10)
+    assert ix.queries_per_launch() == nq
+    assert ix.overflow_redos() >= nq and ix.exact_redos() == 0
+    ix.set_path(4)                                     # tile-group kernels
+    s2, i2 = ix.search(q, 10)
+    ix.set_path(1)                                     # exact path
+    s3, i3 = ix.search(q[:24], 10)
+    ix.set_path(0)
+    assert np.array_equal(i, i2) and bits_equal(s, s2)
+    assert np.array_equal(i[:24], i3) and bits_equal(s[:24], s3)
+    ix.close()
+
+
 def test_wide_scan_with_wild_row_scales(T, oracle):
     """Row scales far from the encoder's (zeros, tiny, huge: the accumulator bound divides by the
     block's largest one) against the oracle; with negative ones mixed in (a foreign snapshot
