@@ -103,9 +103,12 @@ def cpu_baseline(args):
     q = rng.standard_normal((args.batch, dim), dtype=np.float32)
     q /= np.linalg.norm(q, axis=1, keepdims=True)
     search(rot, codes, scales, q[:8], args.k, n_s)   # warm
-    t0 = time.perf_counter()
-    search(rot, codes, scales, q, args.k, n_s)
-    dt = time.perf_counter() - t0
+    ts = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        search(rot, codes, scales, q, args.k, n_s)
+        ts.append(time.perf_counter() - t0)
+    dt = float(np.median(ts))
     pairs_per_s = args.batch * n_s / dt
     what = ("C restatement of the reference's AVX-512 VNNI permute-dot kernel and tiling (search.rs:1392-1567)"
             if vnni else "portable C loop over the reference's arithmetic (host without AVX-512 VNNI)"
@@ -116,7 +119,7 @@ def cpu_baseline(args):
         "cores": threads,
         "kind": "port",
         "sample": f"{args.batch} queries x {n_s} of {args.n} vectors ({dim}-dim, {bits}-bit, k={args.k}), "
-                  f"{dt:.2f} s, scaled by {n_s}/{args.n}; {what}, not the reference binary",
+                  f"median of 5 runs {dt:.2f} s, scaled by {n_s}/{args.n}; {what}, not the reference binary",
     }
     del codes, scales
     if vnni and dim == 1536:
