@@ -416,7 +416,11 @@ struct SamplingSteps {
     size_t size() const { return count; }
     uint32_t operator[](size_t i) const { return step[i]; }
 };
-SamplingSteps sampling_steps(size_t n_blocks, size_t k_floor) {
+// `round_blocks` > 0: the scan kernel works through the blocks in rounds of that many (one per
+// wave of the grid) and a level costs whole rounds whatever it fills of the last one; a level
+// larger than a round is trimmed to whole rounds (its floor gets a little lower, the next level
+// a little longer: at 10M rows 3157 blocks become 2048, one round instead of two).
+SamplingSteps sampling_steps(size_t n_blocks, size_t k_floor, size_t round_blocks = 0) {
     const double n_slots = double(n_blocks * tv::kVecBlock);
     const double first = double(std::max<size_t>(1024, 8 * k_floor));
     SamplingSteps steps;
@@ -426,8 +430,11 @@ SamplingSteps sampling_steps(size_t n_blocks, size_t k_floor) {
         const double ratio = std::pow(n_slots / first, 1.0 / double(levels));
         double sample = first;
         for (int lv = 0; lv < levels && steps.count + 1 < size_t(SamplingSteps::kMax); ++lv, sample *= ratio) {
-            const size_t sample_blocks = std::max<size_t>(1, size_t(sample) / tv::kVecBlock);
-            const size_t step = n_blocks / sample_blocks;
+            size_t sample_blocks = std::max<size_t>(1, size_t(sample) / tv::kVecBlock);
+            if (round_blocks > 0 && sample_blocks > round_blocks) sample_blocks -= sample_blocks % round_blocks;
+            // a trimmed level must not spill into one more round: step rounded up
+            const size_t step = round_blocks > 0 && sample_blocks >= round_blocks ? (n_blocks + sample_blocks - 1) / sample_blocks
+                                                                                  : n_blocks / sample_blocks;
             if (step > 1 && (steps.count == 0 || step < steps.step[steps.count - 1])) steps.step[steps.count++] = uint32_t(step);
         }
     }
@@ -467,7 +474,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
     const size_t n_blocks = (n + tv::kVecBlock - 1) / tv::kVecBlock;
     // sampling levels take the k_floor-th best as the floor: a deeper order statistic is steadier
     const size_t k_floor = std::max<size_t>(k_eff, 16);
-    const SamplingSteps steps = sampling_steps(n_blocks, k_floor);
+    const SamplingSteps steps_plain = sampling_steps(n_blocks, k_floor);
     uint32_t *h_over = ix->h_flags;   // pinned, one flag per query of a chunk
 
     for (size_t q0 = 0; q0 < nq; q0 += kChunkQueries) {
@@ -491,6 +498,8 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             const size_t tile_q = plan.tile_q, n_tiles = plan.n_tiles, cq_pad = plan.cq_pad, seg_stride = plan.seg_stride;
             const bool wide = plan.wide;
             const int grid = plan.grid;
+            const SamplingSteps steps = wide ? sampling_steps(n_blocks, k_floor, size_t(grid) * tv::wide_blocks_per_workgroup(g.nch))
+                                             : steps_plain;
             int prc = ensure_workspace(ix, head.used + plan.need);
             if (prc != TV_OK) return prc;
             Arena ar;

@@ -115,6 +115,7 @@ bool batched_weights_split(int nch);   // which weight order launch_scan_p4_batc
 int wide_min_queries(int nch);
 int wide_grid_blocks(int device);
 hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s);
+int wide_blocks_per_workgroup(int nch);
 
 hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, const int *part_cnt, int total_threads,
                         int qmod, int k, int k_eff, int nq_tile, float *out_scores, int64_t *out_idx,

@@ -524,6 +524,21 @@ int wide_min_queries(int nch) {
     }
 }
 
+// Blocks one workgroup of the instance for this row length holds per round (waves x blocks per
+// wave, or wave pairs); 0 = no instance.
+int wide_blocks_per_workgroup(int nch) {
+    switch (nch) {
+        case 2: return 48;
+        case 4: return 32;
+        case 6: return 24;
+        case 8: case 10: case 12: return 16;
+        case 14: case 16: case 18: case 20: case 22: case 24: return 8;
+        case 28: case 32: case 36: case 40: case 44: case 48: return 4;
+        case 56: case 64: case 72: case 80: case 88: case 96: return 2;
+        default: return 0;
+    }
+}
+
 static size_t wide_lds_bytes(int slot_bytes, int nq, int blk, int ks) {
     const size_t nq_pad = size_t((nq + kQTile - 1) / kQTile) * kQTile;
     return size_t(kWideRing) * slot_bytes + nq_pad * sizeof(WideQuery) + size_t(kWideWaves) * blk * 32 * 4 + 64 +
