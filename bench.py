@@ -34,8 +34,8 @@ sys.path.insert(0, ROOT)
 # HBM bytes one launch of the dominant kernel moves (reads + writes), from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this same command, each scaled by the copy-probe factor (see profiles/).
 MEASURED_TRAFFIC = {
-    ("k_scan_p4_wide", 10_000_000, 1536, 4): 7.7951e9,    # 3,775,900 x 2 KiB fetched + 60,615 KiB written
-    ("k_scan_p4_multi", 10_000_000, 1536, 4): 7.7344e9,   # 3,774,660 x 2 KiB fetched + 3,797 KiB written
+    ("k_scan_p4_wide", 10_000_000, 1536, 4): 7.8248e9,    # 3,775,920 x 2 KiB fetched + 89,521 KiB written
+    ("k_scan_p4_multi", 10_000_000, 1536, 4): 7.7344e9,   # 3,774,660 x 2 KiB fetched + 3,784 KiB written
     ("k_scan_p4", 10_000_000, 1536, 4): 7.7206e9,         # 3,769,810 x 2 KiB fetched + 58 KiB written
     ("k_scan_lut_bt", 10_000_000, 1536, 2): 3.8802e9,     # 1,894,650 x 2 KiB fetched
     ("k_scan_lut", 10_000_000, 1536, 2): 3.8809e9,        # 1,894,970 x 2 KiB fetched
