@@ -165,27 +165,32 @@ def config3_extra(T, torch, build_index, run, args):
     return res
 
 
-def adversarial_extra(T, torch, run, args, normal_ms):
-    """What the candidate-overflow path costs at full size (10M x 1536 4-bit, k=10, 1024 queries) on
-    two insertion orders chosen against it.  (1) a 1000-cluster mixture inserted cluster by cluster,
+def adversarial_extra(T, torch, run, args, normal_ms, ladder):
+    """What the candidate-overflow handling costs at full size (10M x 1536 4-bit, k=10, 1024 queries) on
+    insertion orders chosen against it.  (1) a 1000-cluster mixture inserted cluster by cluster,
     queries next to database rows: every query has thousands of near neighbours in a few hundred
-    consecutive blocks.  (2) an index laid out against the sampler itself: every block the sampling
-    levels of the first pass read (multiples of the level strides) holds rows pointing away from
-    the queries, every other block rows pointing towards them, so the first pass's floors are far
-    too low and every query overflows.  Overflowed queries are scanned once more together (ladder
-    shifted half a stride, from raised floors); what still overflows goes to the exact path."""
+    consecutive blocks.  (2) an index laid out against the sampler itself, with the strides the
+    library reports for this search (tv_debug_sampling_plan): every block any sampling level of the
+    first pass reads holds rows pointing away from the queries, every other block rows pointing
+    towards them, so the full scan starts from a floor far too low, every query overflows, and the
+    batch is scanned again from raised floors (ladder shifted half a stride).  (3) the same with only
+    the first level's blocks poisoned: the second level then lets everything through, overflows, and
+    is repeated on the device from the floor taken from what fitted; the full scan runs once."""
     dev = torch.device("cuda:0")
     n, dim, k, nq = 10_000_000, 1536, 10, 1024
     gen = torch.Generator(device=dev)
     gen.manual_seed(7)
-    out = {"normal_ms_per_step": normal_ms}
+    strides, offsets = ladder
+    out = {"normal_ms_per_step": normal_ms, "ladder_block_strides": [int(x) for x in strides],
+           "repeated_pass_block_offsets": [int(x) for x in offsets]}
 
     def timed(ix, q, steps=3):
         torch.cuda.synchronize()
         os_ = torch.empty(nq, k, device=dev)
         oi = torch.empty(nq, k, dtype=torch.int64, device=dev)
+        ix.level_repeats(track=1)
         ix.search_dev(q.data_ptr(), nq, k, os_.data_ptr(), oi.data_ptr())
-        r0, e0 = ix.overflow_redos(), ix.exact_redos()
+        r0, e0, l0 = ix.overflow_redos(), ix.exact_redos(), ix.level_repeats()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
@@ -194,7 +199,8 @@ def adversarial_extra(T, torch, run, args, normal_ms):
         ms = (time.perf_counter() - t0) / steps * 1e3
         return {"ms_per_step": ms, "vs_normal": ms / normal_ms,
                 "queries_repeated_per_step": (ix.overflow_redos() - r0) / steps,
-                "queries_on_exact_path_per_step": (ix.exact_redos() - e0) / steps}
+                "queries_on_exact_path_per_step": (ix.exact_redos() - e0) / steps,
+                "sampling_levels_repeated_per_step": (ix.level_repeats() - l0) / steps}
 
     # (1) clustered, cluster by cluster
     centres = torch.randn(1000, dim, device=dev, generator=gen)
@@ -215,22 +221,28 @@ def adversarial_extra(T, torch, run, args, normal_ms):
     del ix, v, centres
     torch.cuda.empty_cache()
 
-    # (2) against the sampler: strides of the first pass's sampling levels at this size
+    # (2), (3) against the sampler
     u = torch.randn(dim, device=dev, generator=gen)
     u = u / u.norm()
-    ix = T.NativeIndex(dim, 4)
-    for c0 in range(0, n, 100_000):
-        blocks = torch.arange(c0, c0 + 100_000, device=dev) // 32
-        sampled = (blocks % 98 == 0) | (blocks % 9765 == 0)
-        sign = torch.where(sampled, -1.0, 1.0).unsqueeze(1)
-        v = sign * 0.3 * u + torch.randn(100_000, dim, device=dev, generator=gen) / dim ** 0.5
-        v = (v / v.norm(dim=1, keepdim=True)).contiguous()
-        torch.cuda.synchronize()
-        ix.add_dev(v.data_ptr(), v.shape[0])
     q = u + 0.5 * torch.randn(nq, dim, device=dev, generator=gen) / dim ** 0.5
     q = (q / q.norm(dim=1, keepdim=True)).contiguous()
-    out["laid_out_against_the_sampler"] = timed(ix, q)
-    ix.close()
+    for key, poisoned in (("every_sampling_level_poisoned", strides[:-1]), ("first_sampling_level_poisoned", strides[:1])):
+        ix = T.NativeIndex(dim, 4)
+        for c0 in range(0, n, 100_000):
+            blocks = torch.arange(c0, c0 + 100_000, device=dev) // 32
+            sampled = torch.zeros_like(blocks, dtype=torch.bool)
+            for st in poisoned:
+                sampled |= blocks % int(st) == 0
+            sign = torch.where(sampled, -1.0, 1.0).unsqueeze(1)
+            v = sign * 0.3 * u + torch.randn(100_000, dim, device=dev, generator=gen) / dim ** 0.5
+            v = (v / v.norm(dim=1, keepdim=True)).contiguous()
+            torch.cuda.synchronize()
+            ix.add_dev(v.data_ptr(), v.shape[0])
+        assert [int(x) for x in ix.sampling_plan(nq, k)[0]] == [int(x) for x in strides], "laid out against another ladder"
+        out[key] = timed(ix, q)
+        ix.close()
+        del ix, v
+        torch.cuda.empty_cache()
     return out
 
 
@@ -302,6 +314,7 @@ def main():
         dt = time.perf_counter() - t0
         return dt, scan_ms, launches, ix.queries_per_launch()
 
+    ladder = ix.sampling_plan(args.batch, k)       # block strides of the sampling levels of a batch search here
     alg_bytes = n_blocks * G * 32 + 4 * n          # codes + per-vector scales, one pass
     d_codes, _, code_bytes = ix.device_ptrs()
     read_ms = ix.stream_probe(d_codes, None, code_bytes, reps=5)   # pure read of the same buffer
@@ -316,6 +329,10 @@ def main():
     dt1, scan1_ms, launches1, _ = run(1, max(args.steps, 15), args.warmup)
     b1_steps = max(args.steps, 15)
     b1_launch_s = scan1_ms * 1e-3 / max(launches1, 1)
+    # configuration 2's middle batch: 64 queries are one pass of the tile-group kernel
+    dt64, scan64_ms, launches64, q64_full = run(64, max(args.steps, 10), args.warmup)
+    b64_steps = max(args.steps, 10)
+    b64_launch_s = scan64_ms * 1e-3 / max(launches64, 1)
 
     # End-to-end rate when the boundary hands over host buffers (queries up, results down over PCIe).
     import numpy as np
@@ -334,6 +351,31 @@ def main():
     host_batch_s = median_host_call(q_host, 5)
     host_single_s = median_host_call(q_host[:1], 15)
     host_qps = args.batch / host_batch_s
+    # one call of four chunks (the reference's Python sends 4096-row calls): the chunks are enqueued
+    # back to back and their overflow flags read once
+    q_host4 = make_queries(4 * args.batch).cpu().numpy()
+    host_batch4_s = median_host_call(q_host4, 5)
+    del q_host4
+
+    # Eight caller threads, one query per call (the reference's search is &self and scales with
+    # caller threads): calls that arrive while the index is busy are merged into the next launch.
+    import threading
+    def threads_single(n_threads, calls):
+        qs = [q_host[t:t + 1].copy() for t in range(n_threads)]
+        m0 = ix.merged_calls()
+        def work(t):
+            for _ in range(calls):
+                ix.search(qs[t], k)
+        ths = [threading.Thread(target=work, args=(t,)) for t in range(n_threads)]
+        t0 = time.perf_counter()
+        for th in ths:
+            th.start()
+        for th in ths:
+            th.join()
+        dt_t = time.perf_counter() - t0
+        return n_threads * calls / dt_t, (ix.merged_calls() - m0) / (n_threads * calls)
+    threads_single(8, 3)
+    t8_qps, t8_merged = threads_single(8, 40)
 
     if mode_p:
         kernel = "k_scan_p4_wide" if q_full >= 256 else "k_scan_p4_multi" if q_full > 32 else "k_scan_p4"
@@ -362,9 +404,25 @@ def main():
         "batch1": {"queries_per_s": b1_steps / dt1, "ms_per_query": dt1 / b1_steps * 1e3,
                    "scan_kernel_ms": b1_launch_s * 1e3, "achieved_GBps": alg_bytes / b1_launch_s / 1e9,
                    "frac_of_hbm_peak": alg_bytes / b1_launch_s / 1e9 / 8000.0,
-                   "frac_of_achievable": alg_bytes / b1_launch_s / 1e9 / read_probe},
+                   "frac_of_achievable": alg_bytes / b1_launch_s / 1e9 / read_probe,
+                   "outside_scan_us": (dt1 / b1_steps - b1_launch_s) * 1e6,
+                   "end_to_end_frac_of_hbm_peak": alg_bytes / (dt1 / b1_steps) / 1e9 / 8000.0},
+        "batch64": {"queries_per_s": 64 * b64_steps / dt64, "ms_per_step": dt64 / b64_steps * 1e3,
+                    "queries_per_launch": q64_full, "scan_launch_ms": b64_launch_s * 1e3,
+                    "roofline": {"bound": "hbm", "achieved": alg_bytes / b64_launch_s / 1e9, "peak": 8000.0, "unit": "GB/s",
+                                 "frac": alg_bytes / b64_launch_s / 1e9 / 8000.0,
+                                 "traffic": MEASURED_TRAFFIC.get(("k_scan_p4_multi", n, dim, bits)),
+                                 "kernel": "k_scan_p4_multi" if mode_p else "k_scan_lut",
+                                 "int8_TOPs": 2.0 * min(64, q64_full) * n * dim / b64_launch_s / 1e12 if mode_p else None}},
+        "threads8_batch1": {"queries_per_s": t8_qps, "one_thread_queries_per_s": 1.0 / host_single_s,
+                            "vs_one_thread": t8_qps * host_single_s, "calls_served_by_another_callers_launch": t8_merged,
+                            "note": "8 threads x 40 single-query tv_search calls (host buffers); waiting calls "
+                                    "with the same k and mask are merged into the next launch"},
         "host_buffers": {"queries_per_s": host_qps, "batch_median_ms": host_batch_s * 1e3,
                          "single_query_median_ms": host_single_s * 1e3,
+                         "batch_x4_queries_per_s": 4 * args.batch / host_batch4_s,
+                         "batch_x4_median_ms": host_batch4_s * 1e3,
+                         "batch_x4_vs_batch": (4 * args.batch / host_batch4_s) / host_qps,
                          "note": "tv_search with host query/result buffers (PCIe both ways): median of 5 batch "
                                  "calls and of 15 single-query calls after a warm-up"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s",
@@ -403,7 +461,7 @@ def main():
         torch.cuda.empty_cache()
         out["config3"] = config3_extra(T, torch, build_index, run, args)
         torch.cuda.empty_cache()
-        out["adversarial"] = adversarial_extra(T, torch, run, args, out["ms_per_step"])
+        out["adversarial"] = adversarial_extra(T, torch, run, args, out["ms_per_step"], ladder)
     if args.cpu_sample > 0:
         out["cpu_baseline"] = cpu_baseline(args)
     print(json.dumps(out))

@@ -13,7 +13,11 @@
  * ends in _dev; sizes are element counts.  Functions that mutate an index
  * (upload / append / swap_remove / set_*) need external exclusion, exactly as
  * the reference's `&mut self` methods do; tv_search* may be called from many
- * threads at once (calls on one index are serialised internally).  A process
+ * threads at once: the GPU serves one launch at a time, so calls that arrive
+ * while the index is busy wait, and whoever gets the index next serves every
+ * waiting tv_search (or tv_search_dev) call with the same k and the same mask
+ * pointer together with its own, as one batch; each caller receives exactly the
+ * rows a call of its own would have returned.  A process
  * that has used the library must not fork() and keep using it in the child.
  *
  * Device buffers (_dev entry points, device pointers): the library runs on a
@@ -227,11 +231,29 @@ int tv_debug_queries_per_launch(const tv_index *ix, int *queries);
  * instead of the batched ones; bit 2 keeps them off the all-queries-per-pass
  * kernel only. */
 int tv_debug_set_path(tv_index *ix, int force_full_lists);
+/* The sampling ladder a search for the k best of nq queries (its first chunk of up to 1024) runs
+ * on this index as it stands, unfiltered: block strides of the successive scans, strides[0 ..
+ * *count), the last one 1 (the full scan); level i reads blocks 0, strides[i], 2*strides[i], ...,
+ * and in the repeated pass of queries whose candidates overflowed it starts at block
+ * repeat_offsets[i].  At most cap entries are written (either array may be NULL); *count = 0 means
+ * the search does not sample (large k, or the exact path is forced).  For tests and the bench,
+ * which lay rows out against the ladder. */
+int tv_debug_sampling_plan(const tv_index *ix, size_t nq, size_t k, uint32_t *strides, uint32_t *repeat_offsets,
+                           size_t cap, size_t *count);
+/* A sampling level whose candidates do not fit (its floor came from a level that happened to read
+ * poor rows) runs a second time, on the device, from the floor taken from what did fit.  track = 1
+ * makes searches report such levels (a few hundred bytes more in the flag copy), 0 stops that,
+ * negative leaves it as it is; *count (may be NULL) = levels repeated so far while tracking. */
+int tv_debug_level_repeats(tv_index *ix, int track, size_t *count);
 /* How many queries so far did not finish in the single sampled pass because their
  * candidate buffer overflowed (they are scanned once more, all together, from a raised
  * floor), and how many of those went on to the exact list / select path. */
 int tv_debug_overflow_redos(const tv_index *ix, size_t *count);
 int tv_debug_exact_redos(const tv_index *ix, size_t *count);
+/* How many tv_search / tv_search_dev calls so far were served by another caller's launch: calls
+ * that arrive while the index is busy are merged, by the next caller to get it, with every
+ * waiting call of the same k and mask into one batch. */
+int tv_debug_merged_calls(const tv_index *ix, size_t *count);
 /* Bandwidth probe on the index's stream: reps launches of a pure read-sum over
  * d_src (d_dst NULL) or of a plain copy d_src -> d_dst, bytes each; mean
  * milliseconds per launch.  Calibrates the achievable HBM rate and gives the

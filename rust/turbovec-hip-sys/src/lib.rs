@@ -87,8 +87,11 @@ extern "C" {
     pub fn tv_last_scan_ms(ix: *const tv_index, ms: *mut c_float, launches: *mut c_int) -> c_int;
     pub fn tv_debug_queries_per_launch(ix: *const tv_index, queries: *mut c_int) -> c_int;
     pub fn tv_debug_set_path(ix: *mut tv_index, force_full_lists: c_int) -> c_int;
+    pub fn tv_debug_sampling_plan(ix: *const tv_index, nq: usize, k: usize, strides: *mut u32, repeat_offsets: *mut u32, cap: usize, count: *mut usize) -> c_int;
+    pub fn tv_debug_level_repeats(ix: *mut tv_index, track: c_int, count: *mut usize) -> c_int;
     pub fn tv_debug_overflow_redos(ix: *const tv_index, count: *mut usize) -> c_int;
     pub fn tv_debug_exact_redos(ix: *const tv_index, count: *mut usize) -> c_int;
+    pub fn tv_debug_merged_calls(ix: *const tv_index, count: *mut usize) -> c_int;
     pub fn tv_debug_stream_probe(ix: *mut tv_index, d_src: *const c_void, d_dst: *mut c_void, bytes: usize, reps: c_int, ms_per_rep: *mut c_float) -> c_int;
     pub fn tv_debug_mfma_probe(ix: *mut tv_index, iters: c_int, reps: c_int, ms_per_rep: *mut c_float, ops_per_rep: *mut c_double) -> c_int;
     pub fn tv_index_device_ptrs(ix: *const tv_index, d_codes: *mut *mut c_void, d_scales: *mut *mut c_void, code_bytes: *mut usize) -> c_int;

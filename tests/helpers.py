@@ -49,3 +49,13 @@ def bits_equal(a, b):
     a = np.ascontiguousarray(a, np.float32)
     b = np.ascontiguousarray(b, np.float32)
     return a.shape == b.shape and np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def ladder_for(T, dim, bits, n, nq, k):
+    """(strides, repeat_offsets) of the sampling ladder the library runs for nq queries, k best, on an index of
+    n rows of this shape (the ladder depends on nothing else): asked of a throw-away index of zero rows."""
+    probe = T.NativeIndex(dim, bits)
+    probe.append_rows(np.zeros((n, probe.n_byte_groups), np.uint8), np.zeros(n, np.float32))
+    plan = probe.sampling_plan(nq, k)
+    probe.close()
+    return plan

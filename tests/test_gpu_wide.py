@@ -4,7 +4,7 @@ batches.  Bar: slots and float scores bit-exact."""
 import numpy as np
 import pytest
 
-from helpers import OracleIndex, bits_equal, to_native, unit_gaussian
+from helpers import OracleIndex, bits_equal, ladder_for, to_native, unit_gaussian
 
 pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
@@ -115,9 +115,9 @@ def test_wide_scan_matches_other_paths(T, dim, n, nq):
 
 
 def test_wide_scan_stops_early_when_every_query_overflows(T):
-    """Rows laid out against the sampler for a whole batch: the one sampling level reads every
-    256th block (8192 blocks, k=10: 1024 sampled slots), those blocks hold the opposite of what
-    the queries look for and every other block near-duplicates of it.  Every query's candidate
+    """Rows laid out against the sampler for a whole batch: the one sampling level (8192 blocks,
+    k=10: 1024 sampled slots, every 256th block: the stride is asked of the library) reads blocks
+    that hold the opposite of what the queries look for, every other block near-duplicates of it.  Every query's candidate
     segments fill within a round, the workgroups of the all-queries-per-pass kernel stop claiming
     blocks, and the batch is scanned again from raised floors: the answer equals the exact path's
     and the tile-group kernels', and no query needs the exact path."""
@@ -127,11 +127,14 @@ def test_wide_scan_stops_early_when_every_query_overflows(T):
     gen.manual_seed(5)
     c = torch.randn(dim, device=dev, generator=gen)
     c = c / c.norm()
+    strides, _ = ladder_for(T, dim, 4, n, nq, 10)
+    assert len(strides) == 2 and strides[1] == 1, strides
+    stride = int(strides[0])
     ix = T.NativeIndex(dim, 4)
     for c0 in range(0, n, 65_536):
         m = min(65_536, n - c0)
         block = (torch.arange(c0, c0 + m, device=dev) // 32)
-        sign = torch.where(block % 256 == 0, -1.0, 1.0).unsqueeze(1)
+        sign = torch.where(block % stride == 0, -1.0, 1.0).unsqueeze(1)
         v = sign * c + 0.3 * torch.randn(m, dim, device=dev, generator=gen) / dim ** 0.5
         torch.cuda.synchronize()
         ix.add_dev(v.data_ptr(), m)

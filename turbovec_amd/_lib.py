@@ -33,7 +33,7 @@ EXPORTS = [
     "tv_debug_stream_probe", "tv_debug_mfma_probe", "tv_debug_set_path", "tv_debug_overflow_redos",
     "tv_host_snapshot_len", "tv_host_snapshot_compose", "tv_host_snapshot_info", "tv_host_snapshot_extract",
     "tv_index_to_bytes", "tv_index_from_bytes", "tv_search_dev_noalloc", "tv_noalloc_scratch_bytes",
-    "tv_debug_exact_redos",
+    "tv_debug_exact_redos", "tv_debug_sampling_plan", "tv_debug_merged_calls", "tv_debug_level_repeats",
 ]
 
 _lib = None
@@ -100,6 +100,9 @@ def lib():
     L.tv_debug_set_path.argtypes = [vp, i32]
     L.tv_debug_overflow_redos.argtypes = [vp, C.POINTER(sz)]
     L.tv_debug_exact_redos.argtypes = [vp, C.POINTER(sz)]
+    L.tv_debug_level_repeats.argtypes = [vp, i32, C.POINTER(sz)]
+    L.tv_debug_merged_calls.argtypes = [vp, C.POINTER(sz)]
+    L.tv_debug_sampling_plan.argtypes = [vp, sz, sz, vp, vp, sz, C.POINTER(sz)]
     L.tv_debug_stream_probe.argtypes = [vp, vp, vp, sz, i32, C.POINTER(C.c_float)]
     L.tv_debug_mfma_probe.argtypes = [vp, i32, i32, C.POINTER(C.c_float), C.POINTER(C.c_double)]
     L.tv_host_rotation_tables.argtypes = [i32, vp, vp, C.POINTER(i32), C.POINTER(C.c_float)]
@@ -310,6 +313,26 @@ class NativeIndex:
         c = C.c_size_t(0)
         check(lib().tv_debug_exact_redos(self.h, C.byref(c)))
         return c.value
+
+    def level_repeats(self, track=-1):
+        """Sampling levels that ran twice so far (counted while tracking is on; track=1/0 switches it)."""
+        c = C.c_size_t(0)
+        check(lib().tv_debug_level_repeats(self.h, track, C.byref(c)))
+        return c.value
+
+    def merged_calls(self):
+        """Search calls so far that were served by another caller's launch."""
+        c = C.c_size_t(0)
+        check(lib().tv_debug_merged_calls(self.h, C.byref(c)))
+        return c.value
+
+    def sampling_plan(self, nq, k):
+        """(strides, repeat_offsets) of the sampling ladder a search of nq queries for the k best runs on the
+        index as it stands; the last stride is 1 (the full scan).  Empty when the search does not sample."""
+        strides, offs = np.zeros(32, np.uint32), np.zeros(32, np.uint32)
+        c = C.c_size_t(0)
+        check(lib().tv_debug_sampling_plan(self.h, nq, k, ptr(strides), ptr(offs), 32, C.byref(c)))
+        return strides[:c.value].copy(), offs[:c.value].copy()
 
     def mfma_probe(self, iters=2000, reps=3):
         """int8 operations per second of the batched scan's MFMA loop alone (registers x LDS, no HBM)."""

@@ -2,6 +2,7 @@
 #include "../../include/turbovec_hip.h"
 
 #include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -186,10 +187,25 @@ struct Prepared {
 // Query preparation for one chunk: rotation, TQ+ inverse, table build
 // (turbovec/src/search.rs:3237-3269).  d_q holds nq*dim floats on the device.
 // `split`: permute-dot weights in the order k_scan_p4 reads them (the batched scans take plane order)
-int prepare_queries(tv_index *ix, Arena &ar, const float *d_q, size_t nq, Prepared &out, bool split = true) {
+// `keep_rotated`: the rotated rows are wanted in device memory too (the debug read-back); a search
+// in permute-dot mode does not need them and prepares its queries in a single launch.
+int prepare_queries(tv_index *ix, Arena &ar, const float *d_q, size_t nq, Prepared &out, bool split = true,
+                    bool keep_rotated = false) {
     const tv::Geometry &g = ix->geo;
     const size_t nq_pad = round_up(nq, tv::kQTile);
     const int mode = effective_mode(ix);
+    if (mode == TV_SCORE_P && !keep_rotated) {
+        const bool cal = !ix->tq_shift.empty();
+        out.d_qrot = nullptr;
+        out.d_qscale = ar.take<float>(nq_pad);
+        out.d_qbias = ar.take<float>(nq_pad);
+        out.table_bytes_per_tile = size_t(g.nch) * 2048;
+        out.d_tables = ar.take<uint8_t>(nq_pad / tv::kQTile * out.table_bytes_per_tile);
+        TV_HIP(tv::launch_prep_p(d_q, ix->d_signs, ix->d_perms, g.dim, ix->rot.block, ix->rot.inv_sqrt_block,
+                                 cal ? ix->d_tq_shift : nullptr, cal ? ix->d_tq_scale : nullptr, out.d_tables, out.d_qscale,
+                                 out.d_qbias, g.G, g.nch, ix->cs, nq, nq_pad, split, ix->stream));
+        return TV_OK;
+    }
     float *d_rot = ar.take<float>(nq * g.dim);
     float *d_bias_corr = ar.take<float>(nq_pad);
     TV_HIP(tv::launch_rotate(d_q, d_rot, ix->d_signs, ix->d_perms, g.dim, ix->rot.block, ix->rot.inv_sqrt_block, nq,
@@ -279,6 +295,7 @@ size_t robust_need(const tv_index *ix, size_t cq, size_t k_eff) {
 struct SampledPlan {
     size_t tile_q, n_tiles, cq_pad, seg_stride, need;
     bool wide;
+    int nt_batched;     // query tiles one launch of the tile-group kernels serves (0: one tile per launch)
     int grid;
 };
 SampledPlan sampled_plan(const tv_index *ix, size_t cq) {
@@ -291,6 +308,7 @@ SampledPlan sampled_plan(const tv_index *ix, size_t cq) {
     // large chunks of high-dimensional queries take the wide kernel: all of them in one pass per level
     const int wide_min = tv::wide_min_queries(g.nch);
     p.wide = mode_p && !ix->no_batched && !ix->no_wide && wide_min > 0 && cq >= size_t(wide_min);
+    p.nt_batched = (mode_p && cq > size_t(tv::kQTile) && !ix->no_batched) ? tv::batched_tiles(g.nch) : 0;
     p.grid = p.wide ? tv::wide_grid_blocks(ix->device)
            : mode_p ? tv::scan_grid_blocks(ix->device, mode_p, g.nch, 0, int(p.tile_q))
                     : tv::lut_append_grid(ix->device, g.nch);
@@ -301,22 +319,73 @@ SampledPlan sampled_plan(const tv_index *ix, size_t cq) {
     return p;
 }
 
-// What a chunk keeps at the head of the workspace across its passes: raised floors, the rows to
-// repeat, and their queries packed.
-size_t redo_header_bytes(const tv_index *ix, size_t cq) {
-    return 2 * round_up(cq * 4, 256) + round_up(cq * size_t(ix->geo.dim) * 4, 256);
+// Sampling plan of a search: block strides of the successive append-mode scans,
+// the last one being 1 (the full scan).  The first level reads about `first`
+// slots and, having no floor yet, appends all of them (one short sort); level
+// sizes then grow geometrically to the full index, by a factor chosen so that
+// a level filtered by the floor of the one before appends at most about 4096
+// candidates per query (the floor is the k_floor-th best of the level before,
+// so a level `ratio` times larger keeps about ratio * k_floor).  The sampling
+// levels together read about 1/ratio of the index.
+struct SamplingSteps {
+    static constexpr int kMax = 32;   // levels grow at least fourfold: 2^31 slots need 16 at most
+    uint32_t step[kMax];
+    size_t count = 0;
+    size_t size() const { return count; }
+    uint32_t operator[](size_t i) const { return step[i]; }
+};
+// `round_blocks` > 0: the scan kernel works through the blocks in rounds of that many (one per
+// wave of the grid) and a level costs whole rounds whatever it fills of the last one; a level
+// larger than a round is trimmed to whole rounds (its floor gets a little lower, the next level
+// a little longer: at 10M rows 3157 blocks become 2048, one round instead of two).
+SamplingSteps sampling_steps(size_t n_blocks, size_t k_floor, size_t round_blocks = 0) {
+    const double n_slots = double(n_blocks * tv::kVecBlock);
+    const double first = double(std::max<size_t>(1024, 8 * k_floor));
+    SamplingSteps steps;
+    if (n_slots > 2.0 * first) {
+        const double max_ratio = std::max(4.0, double(tv::kFinalCap / 2) / double(k_floor));
+        const int levels = std::max(1, int(std::ceil(std::log(n_slots / first) / std::log(max_ratio))));
+        const double ratio = std::pow(n_slots / first, 1.0 / double(levels));
+        double sample = first;
+        for (int lv = 0; lv < levels && steps.count + 1 < size_t(SamplingSteps::kMax); ++lv, sample *= ratio) {
+            size_t sample_blocks = std::max<size_t>(1, size_t(sample) / tv::kVecBlock);
+            if (round_blocks > 0 && sample_blocks > round_blocks) sample_blocks -= sample_blocks % round_blocks;
+            // a trimmed level must not spill into one more round: step rounded up
+            const size_t step = round_blocks > 0 && sample_blocks >= round_blocks ? (n_blocks + sample_blocks - 1) / sample_blocks
+                                                                                  : n_blocks / sample_blocks;
+            if (step > 1 && (steps.count == 0 || step < steps.step[steps.count - 1])) steps.step[steps.count++] = uint32_t(step);
+        }
+    }
+    steps.step[steps.count++] = 1;
+    return steps;
 }
 
-// Workspace a chunk of cq queries may need on the sampled path: its own pass, or the repeated
-// pass over a smaller packed batch that falls to another kernel with more candidate segments.
-// Workspace a chunk of cq queries needs on the sampled path: its own pass, and room for the
-// repeated pass to run at least a tile of queries at a time (a smaller packed batch may fall to
-// another kernel with more candidate segments per query; it is then cut into pieces that fit).
+// Queries of one call are processed in chunks of kChunkQueries; the chunks of a group are enqueued
+// back to back and the host reads their overflow flags once, after the group's last chunk.
+constexpr size_t kGroupQueries = 8 * kChunkQueries;
+constexpr size_t kLevelFlagWords = (kGroupQueries / kChunkQueries) * SamplingSteps::kMax;   // per chunk, one word per level
+
+// What a group keeps at the head of the workspace across its passes: per query the overflow flag and
+// the raised floor of the first pass; for the repeated pass the rows to repeat and their queries
+// packed (one chunk's worth at a time); the per-level "candidates did not fit" flags of the pass in
+// flight.
+size_t group_header_bytes(const tv_index *ix, size_t gq) {
+    const size_t cq = std::min(gq, kChunkQueries);
+    return 2 * round_up(gq * 4, 256) + round_up(cq * 4, 256) + round_up(cq * size_t(ix->geo.dim) * 4, 256) +
+           round_up(kLevelFlagWords * 4, 256);
+}
+
+// Workspace the sampled path needs for a call of nq queries: the header of its largest group, the
+// working set of a full chunk (or of the only, smaller one), and room for the repeated pass to run
+// at least a tile of queries at a time (a smaller packed batch may fall to another kernel with
+// more candidate segments per query; it is then cut into pieces that fit).
 constexpr size_t kRepeatPieces[] = {1024, 512, 256, 128, 96, 64, 32};
-size_t sampled_need_worst(const tv_index *ix, size_t cq) {
+size_t sampled_need_worst(const tv_index *ix, size_t nq) {
+    const size_t gq = std::min(nq, kGroupQueries), cq = std::min(nq, kChunkQueries);
     size_t need = sampled_plan(ix, cq).need;
+    if (nq > kChunkQueries && nq % kChunkQueries != 0) need = std::max(need, sampled_plan(ix, nq % kChunkQueries).need);
     need = std::max(need, sampled_plan(ix, std::min<size_t>(cq, tv::kQTile)).need);
-    return need + redo_header_bytes(ix, cq);
+    return need + group_header_bytes(ix, gq);
 }
 
 // Full-range search without sampling: per-lane lists with shared thresholds for
@@ -401,46 +470,35 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
     return TV_OK;
 }
 
-// Sampling plan of a search: block strides of the successive append-mode scans,
-// the last one being 1 (the full scan).  The first level reads about `first`
-// slots and, having no floor yet, appends all of them (one short sort); level
-// sizes then grow geometrically to the full index, by a factor chosen so that
-// a level filtered by the floor of the one before appends at most about 4096
-// candidates per query (the floor is the k_floor-th best of the level before,
-// so a level `ratio` times larger keeps about ratio * k_floor).  The sampling
-// levels together read about 1/ratio of the index.
-struct SamplingSteps {
-    static constexpr int kMax = 32;   // levels grow at least fourfold: 2^31 slots need 16 at most
-    uint32_t step[kMax];
-    size_t count = 0;
-    size_t size() const { return count; }
-    uint32_t operator[](size_t i) const { return step[i]; }
-};
-// `round_blocks` > 0: the scan kernel works through the blocks in rounds of that many (one per
-// wave of the grid) and a level costs whole rounds whatever it fills of the last one; a level
-// larger than a round is trimmed to whole rounds (its floor gets a little lower, the next level
-// a little longer: at 10M rows 3157 blocks become 2048, one round instead of two).
-SamplingSteps sampling_steps(size_t n_blocks, size_t k_floor, size_t round_blocks = 0) {
-    const double n_slots = double(n_blocks * tv::kVecBlock);
-    const double first = double(std::max<size_t>(1024, 8 * k_floor));
-    SamplingSteps steps;
-    if (n_slots > 2.0 * first) {
-        const double max_ratio = std::max(4.0, double(tv::kFinalCap / 2) / double(k_floor));
-        const int levels = std::max(1, int(std::ceil(std::log(n_slots / first) / std::log(max_ratio))));
-        const double ratio = std::pow(n_slots / first, 1.0 / double(levels));
-        double sample = first;
-        for (int lv = 0; lv < levels && steps.count + 1 < size_t(SamplingSteps::kMax); ++lv, sample *= ratio) {
-            size_t sample_blocks = std::max<size_t>(1, size_t(sample) / tv::kVecBlock);
-            if (round_blocks > 0 && sample_blocks > round_blocks) sample_blocks -= sample_blocks % round_blocks;
-            // a trimmed level must not spill into one more round: step rounded up
-            const size_t step = round_blocks > 0 && sample_blocks >= round_blocks ? (n_blocks + sample_blocks - 1) / sample_blocks
-                                                                                  : n_blocks / sample_blocks;
-            if (step > 1 && (steps.count == 0 || step < steps.step[steps.count - 1])) steps.step[steps.count++] = uint32_t(step);
-        }
-    }
-    steps.step[steps.count++] = 1;
-    return steps;
+// Block strides of the sampling ladder a first pass over cq queries runs (the last one is 1).  The
+// all-queries-per-pass kernel works through the blocks in rounds of its grid, and its levels are
+// trimmed to whole rounds.
+//
+// A first pass served by the single-tile permute-dot kernel (up to 32 queries) runs one sampling
+// level only, without a floor: the scan hands over the best row of every block it reads
+// (kModeBest), and the k_floor-th best of those is the floor of the full scan.  The level is
+// sized so that the full scan then appends about 2048 rows per query, and reads at least
+// 8 * k_floor blocks; a quarter of the index or more is not worth sampling.
+constexpr size_t kBestLevelMaxK = 64;
+bool first_level_is_best_of_block(const tv_index *ix, const SampledPlan &plan, size_t k_floor) {
+    return effective_mode(ix) == TV_SCORE_P && !plan.wide && plan.nt_batched == 0 && k_floor <= kBestLevelMaxK;
 }
+SamplingSteps level_strides(const tv_index *ix, const SampledPlan &plan, size_t n_blocks, size_t k_floor, bool repeat) {
+    if (!repeat && first_level_is_best_of_block(ix, plan, k_floor)) {
+        SamplingSteps steps;
+        size_t sample = std::max<size_t>((n_blocks * k_floor + 2047) / 2048, 8 * k_floor);
+        sample = std::min<size_t>(sample, size_t(plan.grid) * (tv::kSegCap / 2));   // a workgroup's blocks fit its segment
+        if (sample * 4 <= n_blocks && n_blocks / sample > 1) steps.step[steps.count++] = uint32_t(n_blocks / sample);
+        steps.step[steps.count++] = 1;
+        return steps;
+    }
+    return plan.wide ? sampling_steps(n_blocks, k_floor, size_t(plan.grid) * tv::wide_blocks_per_workgroup(ix->geo.nch))
+                     : sampling_steps(n_blocks, k_floor);
+}
+// Block offset of a repeated pass's level of stride `step`: it samples other blocks than the pass
+// that misjudged the floor, half a stride in (an even number of blocks, so that mask words stay
+// aligned).
+uint32_t repeat_offset(uint32_t step) { return step >= 4 ? (step / 2) & ~1u : 0u; }
 
 // The seam: search::search over device-resident inputs and outputs.
 //
@@ -474,165 +532,401 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
     const size_t n_blocks = (n + tv::kVecBlock - 1) / tv::kVecBlock;
     // sampling levels take the k_floor-th best as the floor: a deeper order statistic is steadier
     const size_t k_floor = std::max<size_t>(k_eff, 16);
-    const SamplingSteps steps_plain = sampling_steps(n_blocks, k_floor);
-    uint32_t *h_over = ix->h_flags;   // pinned, one flag per query of a chunk
+    uint32_t *h_over = ix->h_flags;   // pinned, one flag per query of a group, then the groups' level flags
+    const bool track_levels = ix->track_levels != 0;
+    // sized once for the whole call, repeated passes included: nothing is reallocated while work is in flight
+    rc = ensure_workspace(ix, sampled_need_worst(ix, nq));
+    if (rc != TV_OK) return rc;
 
-    for (size_t q0 = 0; q0 < nq; q0 += kChunkQueries) {
-        const size_t cq = std::min(kChunkQueries, nq - q0);
-        const float *d_q = d_queries + q0 * g.dim;
-        float *d_os = d_out_scores + q0 * k_eff;
-        int64_t *d_oi = d_out_idx + q0 * k_eff;
-        // sized for the repeated pass too: the head of the workspace must survive between the passes
-        rc = ensure_workspace(ix, sampled_need_worst(ix, cq));
-        if (rc != TV_OK) return rc;
+    for (size_t g0 = 0; g0 < nq; g0 += kGroupQueries) {
+        const size_t gq = std::min(kGroupQueries, nq - g0);
         Arena head;
         head.base = static_cast<uint8_t *>(ix->ws);
-        int *d_raise = head.take<int>(cq);
-        uint32_t *d_rows = head.take<uint32_t>(cq);
-        float *d_redo_q = head.take<float>(cq * g.dim);
+        int *d_raise = head.take<int>(gq);
+        // The overflow flags of the first passes are written by k_final straight into the pinned
+        // host array (device-visible): no copy kernel between the last selection and the host's read.
+        uint32_t *d_over_all = ix->d_flags_host;
+        head.take<uint32_t>(gq);
+        uint32_t *d_rows = head.take<uint32_t>(std::min(gq, kChunkQueries));
+        float *d_redo_q = head.take<float>(std::min(gq, kChunkQueries) * g.dim);
+        uint32_t *d_level_flags_all = head.take<uint32_t>(kLevelFlagWords);
+        size_t n_timed = 0;
 
-        // One pass over `pq_n` queries: the ladder from open floors, or, for the packed batch of
-        // queries to repeat, the ladder again from the floors the pass before raised for them.
-        auto pass = [&](size_t row0, size_t pq_n, bool repeat) -> int {
+        // One pass over `pq_n` queries of the chunk at q0: the ladder from open floors, or, for the
+        // packed batch of queries to repeat (rows d_rows[row0 ..]), the ladder again from the floors
+        // the pass before raised for them.  Enqueues only; the caller synchronises.
+        auto pass = [&](size_t q0, size_t row0, size_t pq_n, bool repeat, bool timed_pass) -> int {
+            const float *d_q = d_queries + q0 * g.dim;
+            float *d_os = d_out_scores + q0 * k_eff;
+            int64_t *d_oi = d_out_idx + q0 * k_eff;
             const SampledPlan plan = sampled_plan(ix, pq_n);
             const size_t tile_q = plan.tile_q, n_tiles = plan.n_tiles, cq_pad = plan.cq_pad, seg_stride = plan.seg_stride;
             const bool wide = plan.wide;
             const int grid = plan.grid;
-            const SamplingSteps steps = wide ? sampling_steps(n_blocks, k_floor, size_t(grid) * tv::wide_blocks_per_workgroup(g.nch))
-                                             : steps_plain;
-            int prc = ensure_workspace(ix, head.used + plan.need);
-            if (prc != TV_OK) return prc;
+            const SamplingSteps steps = level_strides(ix, plan, n_blocks, k_floor, repeat);
+            const bool best_first = !repeat && first_level_is_best_of_block(ix, plan, k_floor) && steps.size() > 1;
+            uint32_t *d_level_flags = d_level_flags_all + ((q0 - g0) / kChunkQueries) * SamplingSteps::kMax;
+            if (head.used + plan.need > ix->ws_bytes) {
+                g_last_error = "internal: workspace smaller than the pass it was sized for";
+                return TV_ERR_BAD_ARGUMENT;
+            }
             Arena ar;
             ar.base = static_cast<uint8_t *>(ix->ws) + head.used;
             int *d_tau = ar.take<int>(n_tiles * tv::kQTile);
-            if (repeat)
-                TV_HIP(tv::launch_gather_redo(d_q, d_rows + row0, d_raise, g.dim, int(tile_q), pq_n, d_redo_q, d_tau, ix->stream));
+            if (repeat) {
+                TV_HIP(tv::launch_gather_redo(d_q, d_rows + row0, d_raise + (q0 - g0), g.dim, int(tile_q), pq_n, d_redo_q, d_tau,
+                                              ix->stream));
+                // every level of a repeated pass filters by a floor: all of their flags start at zero
+                TV_HIP(tv::launch_fill_i32(reinterpret_cast<int *>(d_level_flags), 0, SamplingSteps::kMax, ix->stream));
+            }
             Prepared pq;
-            size_t n_timed = 0;
-            const int nt_batched = (mode_p && pq_n > size_t(tv::kQTile) && !ix->no_batched) ? tv::batched_tiles(g.nch) : 0;
-            prc = prepare_queries(ix, ar, repeat ? d_redo_q : d_q, pq_n, pq,
-                                  !wide && (nt_batched == 0 || tv::batched_weights_split(g.nch)));
+            const int nt_batched = plan.nt_batched;
+            int prc = prepare_queries(ix, ar, repeat ? d_redo_q : d_q, pq_n, pq,
+                                      !wide && (nt_batched == 0 || tv::batched_weights_split(g.nch)));
             if (prc != TV_OK) return prc;
             uint64_t *d_cand = ar.take<uint64_t>(cq_pad * seg_stride * tv::kSegCap);
             uint32_t *d_cnt = ar.take<uint32_t>(cq_pad * seg_stride);
-            uint32_t *d_over = ar.take<uint32_t>(cq_pad);
+            uint32_t *d_over = repeat ? ar.take<uint32_t>(cq_pad) : d_over_all + (q0 - g0);
             // no per-search clears: the first level reads the index's standing array of open floors,
             // every later one the floors k_final wrote, and k_final writes every overflow flag
 
             const int bgrid = tv::batched_grid_blocks(ix->device, g.nch);
+            const bool batched = nt_batched > 0 && !wide;
+            const size_t tiles_per_launch = wide ? n_tiles : batched ? size_t(nt_batched) : 1;
+            if (!repeat) ix->last_queries_per_launch = int(std::min(pq_n, tile_q * tiles_per_launch));
             for (size_t lv = 0; lv < steps.size(); ++lv) {
                 const bool last = lv + 1 == steps.size();
-                // A repeated pass samples other blocks than the pass that misjudged the floor: its
-                // sampling levels start half a stride in (an even number of blocks, so that mask
-                // words stay aligned).  Sampling levels only yield floors, never slots, so the
-                // shifted origin needs no correction downstream.
-                const uint32_t off = (repeat && steps[lv] >= 4) ? (steps[lv] / 2) & ~1u : 0u;
+                // Sampling levels only yield floors, never slots, so the shifted origin of a repeated
+                // pass needs no correction downstream.
+                const uint32_t off = repeat ? repeat_offset(steps[lv]) : 0u;
                 const size_t level_blocks = (n_blocks - off + steps[lv] - 1) / steps[lv];
                 // level 1 appends every slot it reads: two blocks per workgroup fill a segment exactly
                 const int lgrid = int(std::min<size_t>(size_t(grid), std::max<size_t>(1, (level_blocks + 1) / 2)));
-                const bool batched = nt_batched > 0 && !wide;
-                const size_t tiles_per_launch = wide ? n_tiles : batched ? size_t(nt_batched) : 1;
-                if (!repeat) ix->last_queries_per_launch = int(std::min(pq_n, tile_q * tiles_per_launch));
-                int n_seg = lgrid;
-                size_t launch_no = 0;
-                for (size_t t = 0; t < n_tiles; t += tiles_per_launch, ++launch_no) {
-                    tv::ScanArgs a;
-                    fill_scan_args(ix, a);
-                    a.mask = d_mask;
-                    a.tables = pq.d_tables + t * (mode_p ? pq.table_bytes_per_tile : tile_q * size_t(g.nch) * 1024);
-                    a.qscale = pq.d_qscale + t * tile_q;
-                    a.qbias = pq.d_qbias + t * tile_q;
-                    a.nq_tile = int(std::min<size_t>(tile_q * tiles_per_launch, pq_n - t * tile_q));
-                    a.k = 1;
-                    a.gtau = ((lv == 0 && !repeat) ? ix->d_tau_open : d_tau) + t * tv::kQTile;
-                    a.b_step = steps[lv];
-                    if (off) {
-                        a.codes += size_t(off) * g.block_bytes();
-                        a.scales += size_t(off) * tv::kVecBlock;
-                        if (a.mask) a.mask += off / 2;
-                        a.n_blocks -= off;
-                        a.n -= off * tv::kVecBlock;
+                // A sampling level behind the first filters by the floor of the level before; when
+                // that floor was far too low (rows laid out against the sample) its candidates do not
+                // fit, k_final says so in the level's flag, and the level runs once more from the
+                // floor k_final took from what did fit -- launches that do nothing unless the flag
+                // is set.  The full scan then starts from the floor the level was meant to give.
+                uint32_t *lv_flag = (!last && (lv > 0 || repeat)) ? d_level_flags + lv : nullptr;
+                uint32_t *next_flag = (lv + 2 < steps.size()) ? d_level_flags + lv + 1 : nullptr;
+                for (int attempt = 0; attempt < (lv_flag ? 2 : 1); ++attempt) {
+                    const uint32_t *run_if = attempt == 0 ? nullptr : lv_flag;
+                    int n_seg = lgrid;
+                    size_t launch_no = 0;
+                    for (size_t t = 0; t < n_tiles; t += tiles_per_launch, ++launch_no) {
+                        tv::ScanArgs a;
+                        fill_scan_args(ix, a);
+                        a.mask = d_mask;
+                        a.tables = pq.d_tables + t * (mode_p ? pq.table_bytes_per_tile : tile_q * size_t(g.nch) * 1024);
+                        a.qscale = pq.d_qscale + t * tile_q;
+                        a.qbias = pq.d_qbias + t * tile_q;
+                        a.nq_tile = int(std::min<size_t>(tile_q * tiles_per_launch, pq_n - t * tile_q));
+                        a.k = 1;
+                        a.gtau = ((lv == 0 && !repeat) ? ix->d_tau_open : d_tau) + t * tv::kQTile;
+                        a.b_step = steps[lv];
+                        a.run_if = run_if;
+                        if (off) {
+                            a.codes += size_t(off) * g.block_bytes();
+                            a.scales += size_t(off) * tv::kVecBlock;
+                            if (a.mask) a.mask += off / 2;
+                            a.n_blocks -= off;
+                            a.n -= off * tv::kVecBlock;
+                        }
+                        a.cand = d_cand + t * tile_q * seg_stride * tv::kSegCap;
+                        a.cand_cnt = d_cnt + t * tile_q * seg_stride;
+                        a.seg_stride = uint32_t(seg_stride);
+                        const bool timed = timed_pass && last && int(launch_no) < kMaxTimedTiles;
+                        if (timed) TV_HIP(hipEventRecord(ix->ev_start[launch_no], ix->stream));
+                        if (wide) {
+                            n_seg = grid;
+                            TV_HIP(tv::launch_scan_p4_wide(a, n_seg, ix->stream));
+                        } else if (batched) {
+                            n_seg = int(std::min<size_t>(size_t(bgrid), seg_stride));
+                            TV_HIP(tv::launch_scan_p4_batched(a, n_seg, ix->stream));
+                        } else if (mode_p) {
+                            TV_HIP(tv::launch_scan_p4(a, lgrid, (best_first && lv == 0) ? tv::kModeBest : tv::kModeAppend, ix->stream));
+                        } else {
+                            TV_HIP(tv::launch_scan_lut(a, lgrid, tv::kModeAppend, ix->stream));
+                        }
+                        if (timed) TV_HIP(hipEventRecord(ix->ev_stop[launch_no], ix->stream));
                     }
-                    a.cand = d_cand + t * tile_q * seg_stride * tv::kSegCap;
-                    a.cand_cnt = d_cnt + t * tile_q * seg_stride;
-                    a.seg_stride = uint32_t(seg_stride);
-                    const bool timed = timing && !repeat && last && int(launch_no) < kMaxTimedTiles;
-                    if (timed) TV_HIP(hipEventRecord(ix->ev_start[launch_no], ix->stream));
-                    if (wide) {
-                        n_seg = grid;
-                        TV_HIP(tv::launch_scan_p4_wide(a, n_seg, ix->stream));
-                    } else if (batched) {
-                        n_seg = int(std::min<size_t>(size_t(bgrid), seg_stride));
-                        TV_HIP(tv::launch_scan_p4_batched(a, n_seg, ix->stream));
-                    } else if (mode_p) {
-                        TV_HIP(tv::launch_scan_p4(a, lgrid, tv::kModeAppend, ix->stream));
-                    } else {
-                        TV_HIP(tv::launch_scan_lut(a, lgrid, tv::kModeAppend, ix->stream));
-                    }
-                    if (timed) TV_HIP(hipEventRecord(ix->ev_stop[launch_no], ix->stream));
+                    if (last && timed_pass) n_timed = std::min<size_t>(launch_no, size_t(kMaxTimedTiles));
+                    // the first final pass may hand raised floors to a repeated one; the repeated pass
+                    // sends what still does not fit to the exact path
+                    TV_HIP(tv::launch_final(d_cand, d_cnt, uint32_t(n_seg), uint32_t(seg_stride), int(k_eff), int(k_floor),
+                                            int(pq_n), d_os, d_oi, d_over, last ? nullptr : d_tau, int(tile_q),
+                                            (lv > 0 || repeat) ? 1 : 0, (last && !repeat) ? d_raise + (q0 - g0) : nullptr,
+                                            repeat ? d_rows + row0 : nullptr, lv_flag, attempt == 0 ? next_flag : nullptr,
+                                            run_if, ix->stream));
                 }
-                if (last && timing && !repeat) n_timed = std::min<size_t>(launch_no, size_t(kMaxTimedTiles));
-                // the first final pass may hand raised floors to a repeated one; the repeated pass
-                // sends what still does not fit to the exact path
-                TV_HIP(tv::launch_final(d_cand, d_cnt, uint32_t(n_seg), uint32_t(seg_stride), int(k_eff), int(k_floor),
-                                        int(pq_n), d_os, d_oi, d_over, last ? nullptr : d_tau, int(tile_q), (lv > 0 || repeat) ? 1 : 0,
-                                        (last && !repeat) ? d_raise : nullptr, repeat ? d_rows + row0 : nullptr, ix->stream));
             }
-            TV_HIP(hipMemcpyAsync(h_over, d_over, pq_n * sizeof(uint32_t), hipMemcpyDeviceToHost, ix->stream));
-            TV_HIP(hipStreamSynchronize(ix->stream));
-            for (size_t t = 0; t < n_timed; ++t) {
-                float ms = 0.0f;
-                TV_HIP(hipEventElapsedTime(&ms, ix->ev_start[t], ix->ev_stop[t]));
-                ix->last_scan_ms += ms;
-                ix->last_scan_launches += 1;
-            }
+            if (repeat) TV_HIP(hipMemcpyAsync(h_over, d_over, pq_n * sizeof(uint32_t), hipMemcpyDeviceToHost, ix->stream));
             return TV_OK;
         };
 
-        rc = pass(0, cq, false);
-        if (rc != TV_OK) return rc;
-        // Queries whose candidates did not fit (an unlucky sample, adversarial order).  Those that
-        // came back with a raised floor (flag 1) are packed and scanned once more, all together;
-        // what still does not fit then, and what had no floor to raise (flag 2), is redone exactly.
-        uint32_t rows[kChunkQueries];
-        size_t n_rows = 0, n_exact = 0;
-        uint32_t exact_rows[kChunkQueries];
-        for (size_t q = 0; q < cq; ++q) {
-            if (h_over[q] == 1u) rows[n_rows++] = uint32_t(q);
-            else if (h_over[q] != 0u) exact_rows[n_exact++] = uint32_t(q);
+        // first passes of every chunk of the group, back to back; one read of the flags at the end
+        for (size_t c0 = 0; c0 < gq; c0 += kChunkQueries) {
+            rc = pass(g0 + c0, 0, std::min(kChunkQueries, gq - c0), false, timing && c0 == 0);
+            if (rc != TV_OK) return rc;
         }
-        ix->overflow_redos += n_rows + n_exact;
-        if (n_rows) {
-            std::memcpy(h_over, rows, n_rows * sizeof(uint32_t));   // pinned staging for the upload
-            TV_HIP(hipMemcpyAsync(d_rows, h_over, n_rows * sizeof(uint32_t), hipMemcpyHostToDevice, ix->stream));
-            TV_HIP(hipStreamSynchronize(ix->stream));
-            // all of them in one pass when the workspace holds that pass, else in the largest pieces it holds
-            const size_t room = ix->ws_bytes - head.used;
-            for (size_t r0 = 0; r0 < n_rows;) {
-                size_t piece = std::min<size_t>(n_rows - r0, tv::kQTile);
-                for (size_t cand_piece : kRepeatPieces) {
-                    const size_t m = std::min(cand_piece, n_rows - r0);
-                    if (sampled_plan(ix, m).need <= room) { piece = m; break; }
-                }
-                rc = pass(r0, piece, true);
-                if (rc != TV_OK) return rc;
-                for (size_t r = 0; r < piece; ++r)
-                    if (h_over[r] != 0u) exact_rows[n_exact++] = rows[r0 + r];
-                r0 += piece;
+        if (track_levels)
+            TV_HIP(hipMemcpyAsync(h_over + kGroupQueries, d_level_flags_all, kLevelFlagWords * 4, hipMemcpyDeviceToHost, ix->stream));
+        TV_HIP(hipStreamSynchronize(ix->stream));
+        if (track_levels) {
+            // flags of levels the passes above did not use hold whatever the workspace held: count only the used ones
+            for (size_t c0 = 0; c0 < gq; c0 += kChunkQueries) {
+                const SampledPlan plan = sampled_plan(ix, std::min(kChunkQueries, gq - c0));
+                const size_t n_levels = level_strides(ix, plan, n_blocks, k_floor, false).size();
+                for (size_t lv = 1; lv + 1 < n_levels; ++lv)
+                    ix->level_repeats += h_over[kGroupQueries + (c0 / kChunkQueries) * SamplingSteps::kMax + lv] != 0u;
             }
         }
-        std::sort(exact_rows, exact_rows + n_exact);
-        ix->exact_redos += n_exact;
-        for (size_t i = 0; i < n_exact;) {
+        for (size_t t = 0; t < n_timed; ++t) {
+            float ms = 0.0f;
+            TV_HIP(hipEventElapsedTime(&ms, ix->ev_start[t], ix->ev_stop[t]));
+            ix->last_scan_ms += ms;
+            ix->last_scan_launches += 1;
+        }
+        // Queries whose candidates did not fit (an unlucky sample, adversarial order).  Those that
+        // came back with a raised floor (flag 1) are packed and scanned once more, a chunk's worth
+        // together; what still does not fit then, and what had no floor to raise (flag 2), is
+        // redone exactly.
+        std::vector<uint32_t> redo_rows, exact_rows;    // group-relative query numbers
+        for (size_t q = 0; q < gq; ++q) {
+            if (h_over[q] == 1u) redo_rows.push_back(uint32_t(q));
+            else if (h_over[q] != 0u) exact_rows.push_back(uint32_t(q));
+        }
+        ix->overflow_redos += redo_rows.size() + exact_rows.size();
+        const size_t room = ix->ws_bytes - head.used;
+        for (size_t i = 0; i < redo_rows.size();) {
+            // rows of one chunk go together: all of them in one pass when the workspace holds that
+            // pass, else in the largest pieces it holds
+            const size_t chunk = redo_rows[i] / kChunkQueries;
+            size_t e = i;
+            while (e < redo_rows.size() && redo_rows[e] / kChunkQueries == chunk) ++e;
+            size_t piece = std::min<size_t>(e - i, tv::kQTile);
+            for (size_t cand_piece : kRepeatPieces) {
+                const size_t m = std::min(cand_piece, e - i);
+                if (sampled_plan(ix, m).need <= room) { piece = m; break; }
+            }
+            for (size_t r = 0; r < piece; ++r) h_over[r] = redo_rows[i + r] - uint32_t(chunk * kChunkQueries);   // pinned staging
+            TV_HIP(hipMemcpyAsync(d_rows, h_over, piece * sizeof(uint32_t), hipMemcpyHostToDevice, ix->stream));
+            TV_HIP(hipStreamSynchronize(ix->stream));
+            rc = pass(g0 + chunk * kChunkQueries, 0, piece, true, false);
+            if (rc != TV_OK) return rc;
+            TV_HIP(hipStreamSynchronize(ix->stream));
+            for (size_t r = 0; r < piece; ++r)
+                if (h_over[r] != 0u) exact_rows.push_back(redo_rows[i + r]);
+            i += piece;
+        }
+        std::sort(exact_rows.begin(), exact_rows.end());
+        ix->exact_redos += exact_rows.size();
+        for (size_t i = 0; i < exact_rows.size();) {
             size_t e = i + 1;
-            while (e < n_exact && exact_rows[e] == exact_rows[e - 1] + 1) ++e;     // runs of neighbours go together
-            const size_t qa = exact_rows[i], cnt = e - i;
-            rc = search_robust(ix, d_q + qa * g.dim, cnt, k_eff, d_mask, d_os + qa * k_eff, d_oi + qa * k_eff, false);
+            while (e < exact_rows.size() && exact_rows[e] == exact_rows[e - 1] + 1) ++e;     // runs of neighbours go together
+            const size_t qa = g0 + exact_rows[i], cnt = e - i;
+            rc = search_robust(ix, d_queries + qa * g.dim, cnt, k_eff, d_mask, d_out_scores + qa * k_eff, d_out_idx + qa * k_eff,
+                               false);
             if (rc != TV_OK) return rc;
             i = e;
         }
     }
     return TV_OK;
+}
+
+// ---- search calls, merged ----------------------------------------------------------------------
+// The reference's search takes &self and runs on as many caller threads as there are
+// (turbovec/src/lib.rs:22-52, tests/concurrent_search.rs); one GPU serves one launch at a time, and a
+// launch costs the same for one query as for thirty-two.  So calls do not queue up one behind the
+// other: a call registers itself, then waits for the index; whoever gets it next serves every
+// registered call that is compatible with its own (same kind of buffers, same k, same mask) as one
+// batch -- rows of a batch are scored independently, so each caller receives exactly what a call of
+// its own would have returned -- and the others find their results ready when their turn comes.
+constexpr size_t kMergeQueries = 4096;   // queries one merged batch may hold
+
+}  // namespace
+
+struct tv_request {
+    bool host = true;              // tv_search (host buffers) or tv_search_dev (device buffers)
+    const float *q = nullptr;
+    size_t nq = 0, k = 0;
+    const uint64_t *mask = nullptr;
+    size_t mask_arg = 0;           // host: number of mask words; device: the mask's popcount
+    float *out_s = nullptr;
+    int64_t *out_i = nullptr;
+    size_t k_eff = 0;
+    int rc = TV_OK;
+    std::string err;
+    bool done = false;
+};
+
+namespace {
+
+// Serves the calls of `batch` (compatible with each other, at least one) as one search.  The index
+// lock is held.  Returns the status every one of them gets.
+int serve_batch(tv_index *ix, const std::vector<tv_request *> &batch, size_t *k_eff_out) {
+    const tv_request &r0 = *batch[0];
+    TV_HIP(hipSetDevice(ix->device));
+    const size_t n = ix->n, dim = size_t(ix->geo.dim);
+    size_t nq = 0;
+    for (const tv_request *r : batch) nq += r->nq;
+    if (!r0.host) {
+        const size_t n_allowed = r0.mask ? r0.mask_arg : n;
+        if (batch.size() == 1)
+            return search_device(ix, r0.q, nq, r0.k, r0.mask, n_allowed, r0.out_s, r0.out_i, k_eff_out);
+        // several callers' device buffers: gathered into the staging allocation, results scattered back
+        const size_t k_eff = std::min(std::min(r0.k, n), n_allowed);
+        *k_eff_out = k_eff;
+        if (k_eff == 0 || nq == 0) return TV_OK;
+        const size_t q_bytes = round_up(nq * dim * sizeof(float), 256), s_bytes = round_up(nq * k_eff * sizeof(float), 256);
+        const size_t i_bytes = round_up(nq * k_eff * sizeof(int64_t), 256);
+        int rc = ensure_io(ix, q_bytes + s_bytes + i_bytes);
+        if (rc != TV_OK) return rc;
+        uint8_t *base = static_cast<uint8_t *>(ix->io);
+        float *d_q = reinterpret_cast<float *>(base);
+        float *d_s = reinterpret_cast<float *>(base + q_bytes);
+        int64_t *d_i = reinterpret_cast<int64_t *>(base + q_bytes + s_bytes);
+        size_t at = 0;
+        for (const tv_request *r : batch) {
+            if (r->nq) TV_HIP(hipMemcpyAsync(d_q + at * dim, r->q, r->nq * dim * sizeof(float), hipMemcpyDeviceToDevice, ix->stream));
+            at += r->nq;
+        }
+        rc = search_device(ix, d_q, nq, r0.k, r0.mask, n_allowed, d_s, d_i, nullptr);
+        if (rc != TV_OK) return rc;
+        at = 0;
+        for (const tv_request *r : batch) {
+            if (r->nq) {
+                TV_HIP(hipMemcpyAsync(r->out_s, d_s + at * k_eff, r->nq * k_eff * sizeof(float), hipMemcpyDeviceToDevice, ix->stream));
+                TV_HIP(hipMemcpyAsync(r->out_i, d_i + at * k_eff, r->nq * k_eff * sizeof(int64_t), hipMemcpyDeviceToDevice, ix->stream));
+            }
+            at += r->nq;
+        }
+        TV_HIP(hipStreamSynchronize(ix->stream));
+        return TV_OK;
+    }
+    const uint64_t *mask_words = r0.mask;
+    const size_t n_mask_words = r0.mask_arg;
+    size_t n_allowed = n;
+    if (mask_words) {
+        if (n_mask_words != (n + 63) / 64) return TV_ERR_MASK_LENGTH_MISMATCH;
+        n_allowed = 0;  // search.rs:3222-3225; bits at or past n are ignored
+        for (size_t w = 0; w < n_mask_words; ++w) {
+            uint64_t word = mask_words[w];
+            if (w * 64 + 64 > n) word &= (n - w * 64 >= 64) ? ~uint64_t(0) : ((uint64_t(1) << (n - w * 64)) - 1);
+            n_allowed += size_t(__builtin_popcountll(word));
+        }
+    }
+    const size_t k_eff = std::min(std::min(r0.k, n), n_allowed);
+    *k_eff_out = k_eff;
+    ix->last_scan_ms = 0.0f;
+    ix->last_scan_launches = 0;
+    if (k_eff == 0 || nq == 0) return TV_OK;
+    // host staging: queries, mask and results live in the index's own staging allocation (kept
+    // between calls, so a search allocates nothing once it has seen its largest batch), apart
+    // from the per-chunk workspace, which is re-carved freely
+    const size_t q_bytes = round_up(nq * dim * sizeof(float), 256), s_bytes = round_up(nq * k_eff * sizeof(float), 256);
+    const size_t i_bytes = round_up(nq * k_eff * sizeof(int64_t), 256), m_bytes = mask_words ? round_up(n_mask_words * 8, 256) : 0;
+    int rc = ensure_io(ix, q_bytes + s_bytes + i_bytes + m_bytes);
+    if (rc != TV_OK) return rc;
+    uint8_t *base = static_cast<uint8_t *>(ix->io);
+    float *d_q = reinterpret_cast<float *>(base);
+    float *d_s = reinterpret_cast<float *>(base + q_bytes);
+    int64_t *d_i = reinterpret_cast<int64_t *>(base + q_bytes + s_bytes);
+    uint64_t *d_m = mask_words ? reinterpret_cast<uint64_t *>(base + q_bytes + s_bytes + i_bytes) : nullptr;
+    size_t at = 0;
+    for (const tv_request *r : batch) {
+        if (r->nq && hipMemcpyAsync(d_q + at * dim, r->q, r->nq * dim * sizeof(float), hipMemcpyHostToDevice, ix->stream) != hipSuccess) {
+            g_last_error = "host to device copy failed";
+            return TV_ERR_HIP;
+        }
+        at += r->nq;
+    }
+    if (mask_words && hipMemcpyAsync(d_m, mask_words, n_mask_words * 8, hipMemcpyHostToDevice, ix->stream) != hipSuccess) {
+        g_last_error = "host to device copy failed";
+        return TV_ERR_HIP;
+    }
+    rc = search_device(ix, d_q, nq, r0.k, d_m, n_allowed, d_s, d_i, nullptr);
+    if (rc != TV_OK) return rc;
+    at = 0;
+    for (const tv_request *r : batch) {
+        if (r->nq && (hipMemcpyAsync(r->out_s, d_s + at * k_eff, r->nq * k_eff * sizeof(float), hipMemcpyDeviceToHost, ix->stream) != hipSuccess ||
+                      hipMemcpyAsync(r->out_i, d_i + at * k_eff, r->nq * k_eff * sizeof(int64_t), hipMemcpyDeviceToHost, ix->stream) != hipSuccess)) {
+            g_last_error = "device to host copy failed";
+            return TV_ERR_HIP;
+        }
+        at += r->nq;
+    }
+    if (hipStreamSynchronize(ix->stream) != hipSuccess) {
+        g_last_error = "device to host copy failed";
+        return TV_ERR_HIP;
+    }
+    return TV_OK;
+}
+
+bool compatible(const tv_request &a, const tv_request &b) {
+    return a.host == b.host && a.k == b.k && a.mask == b.mask && a.mask_arg == b.mask_arg;
+}
+
+// How long a caller that is about to serve waits for the callers of the batch before to come back
+// with their next call (they were all released at the same moment and are a few microseconds of
+// host code away from asking again).  Only after a batch that did merge calls.
+constexpr auto kGatherWait = std::chrono::microseconds(150);
+
+int search_merged(tv_index *ix, tv_request &r) {
+    std::vector<tv_request *> batch;
+    {
+        std::unique_lock<std::mutex> reg(ix->waiting_mu);
+        ix->waiting.push_back(&r);
+        ix->waiting_cv.notify_all();       // a serving caller gathering its batch may be waiting for this one
+        for (;;) {
+            if (r.done) {                  // served by another caller's launch
+                if (r.rc != TV_OK) g_last_error = r.err;
+                return r.rc;
+            }
+            if (!ix->serving) break;
+            ix->waiting_cv.wait(reg);
+        }
+        ix->serving = true;
+        // Callers in a loop come back together: when the batch before held several calls, give the
+        // same number a moment to register again instead of serving this one alone and all of them
+        // in the launch after.
+        if (ix->last_batch_calls > 1) {
+            const auto deadline = std::chrono::steady_clock::now() + kGatherWait;
+            while (ix->waiting.size() < ix->last_batch_calls)
+                if (ix->waiting_cv.wait_until(reg, deadline) == std::cv_status::timeout) break;
+        }
+        // this call first, then the compatible ones in order of arrival, up to the batch limit
+        batch.push_back(&r);
+        size_t total = r.nq;
+        std::vector<tv_request *> rest;
+        for (tv_request *w : ix->waiting) {
+            if (w == &r) continue;
+            if (compatible(*w, r) && total + w->nq <= kMergeQueries) { batch.push_back(w); total += w->nq; }
+            else rest.push_back(w);
+        }
+        ix->waiting.swap(rest);
+    }
+    size_t k_eff = 0;
+    int rc;
+    {
+        std::lock_guard<std::mutex> lock(ix->mu);   // against the entry points that change the index
+        g_last_error.clear();
+        rc = serve_batch(ix, batch, &k_eff);
+    }
+    {
+        std::lock_guard<std::mutex> reg(ix->waiting_mu);
+        for (tv_request *w : batch) {
+            w->rc = rc;
+            w->k_eff = k_eff;
+            if (rc != TV_OK) w->err = g_last_error;
+            w->done = true;
+        }
+        ix->merged_calls += batch.size() - 1;
+        ix->last_batch_calls = batch.size();
+        ix->serving = false;
+    }
+    ix->waiting_cv.notify_all();
+    return rc;
 }
 
 }  // namespace
@@ -701,7 +995,11 @@ int tv_index_create(int dim, int bits, int device, tv_index **out) {
             rc = TV_ERR_HIP;
             break;
         }
-        if (hipHostMalloc(reinterpret_cast<void **>(&ix->h_flags), kChunkQueries * sizeof(uint32_t), hipHostMallocDefault) != hipSuccess) {
+        if (hipHostMalloc(reinterpret_cast<void **>(&ix->h_flags), (kGroupQueries + kLevelFlagWords) * sizeof(uint32_t), hipHostMallocMapped) != hipSuccess) {
+            rc = TV_ERR_HIP;
+            break;
+        }
+        if (hipHostGetDevicePointer(reinterpret_cast<void **>(&ix->d_flags_host), ix->h_flags, 0) != hipSuccess) {
             rc = TV_ERR_HIP;
             break;
         }
@@ -990,10 +1288,8 @@ int tv_index_swap_remove(tv_index *ix, size_t idx) {
     return TV_OK;
 }
 
-int tv_index_download_seq(const tv_index *cix, uint8_t *seq_out, float *scales_out) {
-    tv_index *ix = const_cast<tv_index *>(cix);
-    if (!ix) return TV_ERR_BAD_ARGUMENT;
-    std::lock_guard<std::mutex> lock(ix->mu);
+// The index's lock is held by the caller.
+static int download_seq_locked(tv_index *ix, uint8_t *seq_out, float *scales_out) {
     TV_HIP(hipSetDevice(ix->device));
     const tv::Geometry &g = ix->geo;
     const size_t n_blocks = (ix->n + tv::kVecBlock - 1) / tv::kVecBlock;
@@ -1014,6 +1310,13 @@ int tv_index_download_seq(const tv_index *cix, uint8_t *seq_out, float *scales_o
         TV_HIP(hipStreamSynchronize(ix->stream));
     }
     return TV_OK;
+}
+
+int tv_index_download_seq(const tv_index *cix, uint8_t *seq_out, float *scales_out) {
+    tv_index *ix = const_cast<tv_index *>(cix);
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    return download_seq_locked(ix, seq_out, scales_out);
 }
 
 size_t tv_index_len(const tv_index *ix) { return ix ? ix->n : 0; }
@@ -1048,10 +1351,14 @@ int tv_pack_mask(const uint8_t *mask_bytes, size_t n, uint64_t *words_out, size_
 int tv_search_dev(tv_index *ix, const float *d_queries, size_t nq, size_t k, const uint64_t *d_mask_words,
                   size_t n_allowed, float *d_out_scores, int64_t *d_out_indices, size_t *out_k_eff) {
     if (!ix) return TV_ERR_BAD_ARGUMENT;
-    std::lock_guard<std::mutex> lock(ix->mu);
-    TV_HIP(hipSetDevice(ix->device));
-    if (!d_mask_words) n_allowed = ix->n;
-    return search_device(ix, d_queries, nq, k, d_mask_words, n_allowed, d_out_scores, d_out_indices, out_k_eff);
+    tv_request r;
+    r.host = false;
+    r.q = d_queries; r.nq = nq; r.k = k;
+    r.mask = d_mask_words; r.mask_arg = d_mask_words ? n_allowed : 0;
+    r.out_s = d_out_scores; r.out_i = d_out_indices;
+    const int rc = search_merged(ix, r);
+    if (out_k_eff) *out_k_eff = r.k_eff;
+    return rc;
 }
 
 size_t tv_noalloc_scratch_bytes(void) { return kScratchBytes; }
@@ -1069,7 +1376,7 @@ int tv_search_dev_noalloc(tv_index *ix, const float *d_queries, size_t nq, size_
     if (k_eff != 0 && nq != 0) {
         const size_t cq = std::min(nq, kChunkQueries);
         need = robust_need(ix, cq, k_eff);
-        if (k_eff <= size_t(tv::kMaxSampledK) && !ix->force_robust) need = std::max(need, sampled_need_worst(ix, cq));
+        if (k_eff <= size_t(tv::kMaxSampledK) && !ix->force_robust) need = std::max(need, sampled_need_worst(ix, nq));
     }
     if (need > kScratchBytes) {
         g_last_error = "tv_search_dev_noalloc: " + std::to_string(nq) + " queries, k=" + std::to_string(k) + " over " +
@@ -1094,51 +1401,14 @@ int tv_search_dev_noalloc(tv_index *ix, const float *d_queries, size_t nq, size_
 int tv_search(tv_index *ix, const float *queries, size_t nq, size_t k, const uint64_t *mask_words,
               size_t n_mask_words, float *out_scores, int64_t *out_indices, size_t *out_k_eff) {
     if (!ix || (nq && !queries)) return TV_ERR_BAD_ARGUMENT;
-    std::lock_guard<std::mutex> lock(ix->mu);
-    TV_HIP(hipSetDevice(ix->device));
-    const size_t n = ix->n;
-    size_t n_allowed = n;
-    if (mask_words) {
-        if (n_mask_words != (n + 63) / 64) return TV_ERR_MASK_LENGTH_MISMATCH;
-        n_allowed = 0;  // search.rs:3222-3225; bits at or past n are ignored
-        for (size_t w = 0; w < n_mask_words; ++w) {
-            uint64_t word = mask_words[w];
-            if (w * 64 + 64 > n) word &= (n - w * 64 >= 64) ? ~uint64_t(0) : ((uint64_t(1) << (n - w * 64)) - 1);
-            n_allowed += size_t(__builtin_popcountll(word));
-        }
-    }
-    const size_t k_eff = std::min(std::min(k, n), n_allowed);
-    if (out_k_eff) *out_k_eff = k_eff;
-    ix->last_scan_ms = 0.0f;
-    ix->last_scan_launches = 0;
-    if (k_eff == 0 || nq == 0) return TV_OK;
-    // host staging: queries, mask and results live in the index's own staging allocation (kept
-    // between calls, so a search allocates nothing once it has seen its largest batch), apart
-    // from the per-chunk workspace, which is re-carved freely
-    const size_t dim = size_t(ix->geo.dim);
-    const size_t q_bytes = round_up(nq * dim * sizeof(float), 256), s_bytes = round_up(nq * k_eff * sizeof(float), 256);
-    const size_t i_bytes = round_up(nq * k_eff * sizeof(int64_t), 256), m_bytes = mask_words ? round_up(n_mask_words * 8, 256) : 0;
-    int rc = ensure_io(ix, q_bytes + s_bytes + i_bytes + m_bytes);
-    if (rc != TV_OK) return rc;
-    uint8_t *base = static_cast<uint8_t *>(ix->io);
-    float *d_q = reinterpret_cast<float *>(base);
-    float *d_s = reinterpret_cast<float *>(base + q_bytes);
-    int64_t *d_i = reinterpret_cast<int64_t *>(base + q_bytes + s_bytes);
-    uint64_t *d_m = mask_words ? reinterpret_cast<uint64_t *>(base + q_bytes + s_bytes + i_bytes) : nullptr;
-    if (hipMemcpyAsync(d_q, queries, nq * dim * sizeof(float), hipMemcpyHostToDevice, ix->stream) != hipSuccess ||
-        (mask_words && hipMemcpyAsync(d_m, mask_words, n_mask_words * 8, hipMemcpyHostToDevice, ix->stream) != hipSuccess)) {
-        g_last_error = "host to device copy failed";
-        return TV_ERR_HIP;
-    }
-    rc = search_device(ix, d_q, nq, k, d_m, n_allowed, d_s, d_i, nullptr);
-    if (rc != TV_OK) return rc;
-    if (hipMemcpyAsync(out_scores, d_s, nq * k_eff * sizeof(float), hipMemcpyDeviceToHost, ix->stream) != hipSuccess ||
-        hipMemcpyAsync(out_indices, d_i, nq * k_eff * sizeof(int64_t), hipMemcpyDeviceToHost, ix->stream) != hipSuccess ||
-        hipStreamSynchronize(ix->stream) != hipSuccess) {
-        g_last_error = "device to host copy failed";
-        return TV_ERR_HIP;
-    }
-    return TV_OK;
+    tv_request r;
+    r.host = true;
+    r.q = queries; r.nq = nq; r.k = k;
+    r.mask = mask_words; r.mask_arg = mask_words ? n_mask_words : 0;
+    r.out_s = out_scores; r.out_i = out_indices;
+    const int rc = search_merged(ix, r);
+    if (out_k_eff) *out_k_eff = r.k_eff;
+    return rc;
 }
 
 int tv_debug_scan(tv_index *ix, const float *queries, size_t nq, int32_t *acc_out, float *scores_out) {
@@ -1198,7 +1468,7 @@ int tv_debug_prepare(tv_index *ix, const float *queries, size_t nq, float *q_rot
     float *d_q = ar.take<float>(nq * g.dim);
     TV_HIP(hipMemcpyAsync(d_q, queries, nq * g.dim * sizeof(float), hipMemcpyHostToDevice, ix->stream));
     Prepared pq;
-    rc = prepare_queries(ix, ar, d_q, nq, pq);
+    rc = prepare_queries(ix, ar, d_q, nq, pq, true, true);
     if (rc != TV_OK) return rc;
     if (q_rot_out) TV_HIP(hipMemcpyAsync(q_rot_out, pq.d_qrot, nq * g.dim * 4, hipMemcpyDeviceToHost, ix->stream));
     if (scale_out) TV_HIP(hipMemcpyAsync(scale_out, pq.d_qscale, nq * 4, hipMemcpyDeviceToHost, ix->stream));
@@ -1280,9 +1550,12 @@ int tv_host_snapshot_extract(const uint8_t *bytes, size_t len, float *boundaries
     return TV_OK;
 }
 
-int tv_index_to_bytes(const tv_index *ix, const uint64_t *ids, int format, uint8_t *out, size_t cap, size_t *len) {
+int tv_index_to_bytes(const tv_index *cix, const uint64_t *ids, int format, uint8_t *out, size_t cap, size_t *len) {
+    tv_index *ix = const_cast<tv_index *>(cix);
     if (!ix || !len || (format != 6 && format != 7)) return TV_ERR_BAD_ARGUMENT;
     const int kind = ids ? 1 : 0;
+    // one lock over size, download and compose: the image is of one state of the index
+    std::lock_guard<std::mutex> lock(ix->mu);
     const size_t n = ix->n, n_calib = ix->tq_shift.size();
     *len = tv::snapshot_len(format, ix->geo.dim, ix->geo.bits, kind, n_calib, n);
     if (!out) return TV_OK;
@@ -1290,7 +1563,7 @@ int tv_index_to_bytes(const tv_index *ix, const uint64_t *ids, int format, uint8
     const size_t nb = (n + 31) / 32;
     std::vector<uint8_t> seq(nb * size_t(ix->geo.G) * 32);
     std::vector<float> scales(n);
-    int rc = tv_index_download_seq(ix, seq.data(), scales.data());
+    int rc = download_seq_locked(ix, seq.data(), scales.data());
     if (rc != TV_OK) return rc;
     const tv::SnapshotParts s{kind, ix->geo.dim, ix->geo.bits, ix->cb.boundaries.data(), ix->cb.centroids.data(),
                               n_calib, ix->tq_shift.data(), ix->tq_scale.data(), seq.data(), n, scales.data(), ids};
@@ -1370,9 +1643,37 @@ int tv_debug_mfma_probe(tv_index *ix, int iters, int reps, float *ms_per_rep, do
 
 int tv_debug_set_path(tv_index *ix, int force_full_lists) {
     if (!ix) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
     ix->force_robust = (force_full_lists & 1) != 0;
     ix->no_batched = (force_full_lists & 2) != 0;
     ix->no_wide = (force_full_lists & 4) != 0;
+    return TV_OK;
+}
+
+int tv_debug_sampling_plan(const tv_index *cix, size_t nq, size_t k, uint32_t *strides, uint32_t *repeat_offsets, size_t cap,
+                           size_t *count) {
+    tv_index *ix = const_cast<tv_index *>(cix);
+    if (!ix || !count) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    *count = 0;
+    const size_t k_eff = std::min(k, ix->n);
+    if (k_eff == 0 || nq == 0 || k_eff > size_t(tv::kMaxSampledK) || ix->force_robust) return TV_OK;   // no ladder
+    const size_t n_blocks = (ix->n + tv::kVecBlock - 1) / tv::kVecBlock;
+    const SampledPlan plan = sampled_plan(ix, std::min(nq, kChunkQueries));
+    const SamplingSteps steps = level_strides(ix, plan, n_blocks, std::max<size_t>(k_eff, 16), false);
+    *count = steps.size();
+    for (size_t i = 0; i < steps.size() && i < cap; ++i) {
+        if (strides) strides[i] = steps[i];
+        if (repeat_offsets) repeat_offsets[i] = repeat_offset(steps[i]);
+    }
+    return TV_OK;
+}
+
+int tv_debug_level_repeats(tv_index *ix, int track, size_t *count) {
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    if (track >= 0) ix->track_levels = track;
+    if (count) *count = ix->level_repeats;
     return TV_OK;
 }
 
@@ -1385,6 +1686,14 @@ int tv_debug_overflow_redos(const tv_index *ix, size_t *count) {
 int tv_debug_exact_redos(const tv_index *ix, size_t *count) {
     if (!ix || !count) return TV_ERR_BAD_ARGUMENT;
     *count = ix->exact_redos;
+    return TV_OK;
+}
+
+int tv_debug_merged_calls(const tv_index *cix, size_t *count) {
+    tv_index *ix = const_cast<tv_index *>(cix);
+    if (!ix || !count) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> reg(ix->waiting_mu);
+    *count = ix->merged_calls;
     return TV_OK;
 }
 

@@ -132,6 +132,12 @@ __device__ __forceinline__ uint32_t levels_of(uint32_t nib, uint32_t t0, uint32_
 }
 
 
+// A conditional launch: true when the flag it depends on says there is nothing to do.  The flag is
+// uniform over the grid and written by an earlier launch of the same stream.
+__device__ __forceinline__ bool launch_switched_off(const uint32_t *run_if) {
+    return run_if != nullptr && *reinterpret_cast<const volatile uint32_t *>(run_if) == 0u;
+}
+
 // Compile-time loop: f(IntC<0>{}), ..., f(IntC<N-1>{}), for bodies that index register arrays.
 template <int V> struct IntC { static constexpr int value = V; };
 template <int N, int I = 0, typename F>

@@ -4,6 +4,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <condition_variable>
 #include <mutex>
 #include <vector>
 
@@ -24,7 +25,8 @@ constexpr int kTimedLaunches = 32;  // scan launches of one search that are time
 // What a scan launch does with the scores it computes.
 enum { kModeLists = 0,   // per-lane top-k lists (written out for k_merge)
        kModeDump = 1,    // every score (and accumulator) to dense rows
-       kModeAppend = 2   // every allowed slot scoring >= the query's fixed floor to a candidate buffer
+       kModeAppend = 2,  // every allowed slot scoring >= the query's fixed floor to a candidate buffer
+       kModeBest = 3     // per scanned block and query, the best allowed slot to the candidate buffer (no floor)
 };
 
 // Native device layout of the codes ("vm32"): the byte of (block b, group g,
@@ -65,6 +67,7 @@ struct ScanArgs {
     uint64_t *cand;            // append mode: [nq_tile][seg_stride][kSegCap] sort keys, one segment per workgroup
     uint32_t *cand_cnt;        // append mode: [nq_tile][seg_stride] counts (above kSegCap: that segment overflowed)
     uint32_t seg_stride;       // segments allocated per query (>= grid of the launch)
+    const uint32_t *run_if;    // append mode: when given and *run_if == 0 the launch does nothing (a level's conditional repeat)
 };
 
 // ---- launchers (tv_kernels.hip) ----
@@ -90,6 +93,11 @@ hipError_t launch_calibrate(const float *d_qrot, float *d_qcal, float *d_bias_co
 hipError_t launch_build_p(const float *d_qcal, const float *d_bias_corr, uint8_t *d_wfrag, float *d_qscale,
                           float *d_qbias, int dim, int G, int nch, float cs, size_t nq, size_t nq_padded,
                           bool split, hipStream_t s);
+// Rotation, TQ+ inverse (d_shift / d_scale null: none) and permute-dot weights in one launch.
+hipError_t launch_prep_p(const float *d_q, const float *d_signs, const uint32_t *d_perms, int dim, int block,
+                         float inv_sqrt_block, const float *d_shift, const float *d_scale, uint8_t *d_wfrag,
+                         float *d_qscale, float *d_qbias, int G, int nch, float cs, size_t nq, size_t nq_padded, bool split,
+                         hipStream_t s);
 hipError_t launch_build_lut(const float *d_qcal, const float *d_bias_corr, const float *d_centroids, uint8_t *d_lut,
                             float *d_qscale, float *d_qbias, int dim, int bits, int G, int nch, size_t nq,
                             size_t nq_padded, hipStream_t s);
@@ -127,10 +135,13 @@ hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, cons
 // candidates leaves the floor already there in place instead of opening it).  A final pass that
 // overflows writes flag 1 and a raised floor to raise_out[q] when raise_out is given (flag 2 and
 // nothing otherwise); row_map, when given, names the output row of each query.
+// level_over (sampling levels): set to 1 when some query's candidates of this level did not all fit
+// (its floor then comes from a subset and may be far too low); clear_flag: a word this launch resets
+// to 0 (the flag of the level after); run_if: when given and *run_if == 0 the launch does nothing.
 hipError_t launch_final(const uint64_t *cand, const uint32_t *cand_cnt, uint32_t n_seg, uint32_t seg_stride,
                         int k_eff, int k_floor, int nq, float *out_scores, int64_t *out_idx, uint32_t *overflow,
                         int *tau_out, int tau_stride_q, int keep_floor, int *raise_out, const uint32_t *row_map,
-                        hipStream_t s);
+                        uint32_t *level_over, uint32_t *clear_flag, const uint32_t *run_if, hipStream_t s);
 // Packs the queries rows[0..n_redo) of a chunk and their raised floors for one more full scan.
 hipError_t launch_gather_redo(const float *d_q, const uint32_t *d_rows, const int *d_raised, int dim, int tile_q,
                               size_t n_redo, float *d_q_out, int *d_tau_out, hipStream_t s);
@@ -143,6 +154,8 @@ hipError_t launch_select_topk(const float *d_scores, size_t n, int nq_tile, size
 size_t select_tmp_keys(size_t k_eff);
 
 }  // namespace tv
+
+struct tv_request;   // a search call waiting for the index (tv_api.hip)
 
 // The opaque handle of the C ABI.
 struct tv_index {
@@ -169,6 +182,15 @@ struct tv_index {
     size_t cap_blocks = 0;
     size_t n = 0;
 
+    // Search calls that arrived while another held the index: whoever takes `mu` next serves every
+    // waiting call that asks for the same k under the same mask together with its own, as one batch.
+    std::mutex waiting_mu;
+    std::condition_variable waiting_cv;   // a call registered, or a batch was served
+    std::vector<tv_request *> waiting;
+    bool serving = false;          // some caller is serving a batch right now
+    size_t last_batch_calls = 0;   // calls in the batch served last: how many callers to expect again shortly
+    size_t merged_calls = 0;       // calls that were served by another caller's launch
+
     // per-search workspace, grown on demand, guarded by mu
     mutable std::mutex mu;
     void *ws = nullptr;
@@ -177,7 +199,8 @@ struct tv_index {
     size_t ws_bytes = 0;
     bool ws_fixed = false;         // ws is a lent buffer of fixed size (tv_search_dev_noalloc): never reallocated
     void *scratch = nullptr;       // this device's copy of the library's static scratch array
-    uint32_t *h_flags = nullptr;   // pinned host memory: the overflow flags of one chunk of queries, then the rows to repeat
+    uint32_t *h_flags = nullptr;   // pinned host memory: the overflow flags of one group of chunks, then the rows to repeat
+    uint32_t *d_flags_host = nullptr;   // the device's address of h_flags
     size_t exact_redos = 0;        // queries that went on to the exact path
     float last_scan_ms = 0.0f;
     int last_scan_launches = 0;
@@ -186,4 +209,6 @@ struct tv_index {
     int no_batched = 0;            // test hook: one query tile per scan launch even for large batches
     int no_wide = 0;               // test hook: large batches go through the tile-group kernels, not the wide one
     size_t overflow_redos = 0;     // queries redone because their candidate buffer overflowed
+    int track_levels = 0;          // test hook: read the per-level flags back with the overflow flags and count them
+    size_t level_repeats = 0;      // sampling levels that ran a second time because their candidates did not fit
 };

@@ -250,6 +250,91 @@ __global__ __launch_bounds__(256) void k_build_p(const float *__restrict__ qcal,
     }
 }
 
+// Query preparation of the permute-dot mode in one launch, one workgroup per query: k_rotate,
+// k_calibrate and k_build_p back to back with the row kept in LDS between them -- the same
+// operations on the same values in the same order, so the same bits (search.rs:3237-3269).  A
+// single query's preparation is three dependent launches' worth of latency otherwise.
+__global__ __launch_bounds__(256) void k_prep_p(const float *__restrict__ q, const float *__restrict__ signs,
+                                                const uint32_t *__restrict__ perms, int dim, int block,
+                                                float inv_sqrt_block, const float *__restrict__ shift,
+                                                const float *__restrict__ scale, uint8_t *__restrict__ wfrag,
+                                                float *__restrict__ qscale, float *__restrict__ qbias, int G, int nch,
+                                                float cs, size_t nq, bool split) {
+    extern __shared__ float rot_lds[];
+    __shared__ float red[4];
+    __shared__ float s_bias;
+    float *A = rot_lds;
+    float *B = rot_lds + dim;
+    const size_t qi = blockIdx.x;
+    const size_t tile = qi / kQTile;
+    const int n = int(qi % kQTile);
+    uint8_t *base = wfrag + tile * size_t(nch) * 2048;
+    const int t = threadIdx.x;
+    if (qi >= nq) {  // padding query of the last tile: zero weights
+        for (int g = t; g < nch * 32; g += 256) {
+            base[wfrag_offset(g, n, 0, split)] = 0;
+            base[wfrag_offset(g, n, 1, split)] = 0;
+        }
+        if (t == 0) { qscale[qi] = 0.0f; qbias[qi] = 0.0f; }
+        return;
+    }
+    const float *src = q + qi * size_t(dim);
+    for (int i = t; i < dim; i += 256) A[i] = src[perms[i]] * signs[i];
+    __syncthreads();
+    for (int len = 1; len < block; len <<= 1) {
+        for (int p = t; p < dim / 2; p += 256) {
+            const int j = 2 * p - (p & (len - 1));
+            const float a = A[j], b = A[j + len];
+            A[j] = a + b;
+            A[j + len] = a - b;
+        }
+        __syncthreads();
+    }
+    for (int i = t; i < dim; i += 256) B[i] = (A[perms[dim + i]] * inv_sqrt_block) * signs[dim + i];
+    __syncthreads();
+    for (int len = 1; len < block; len <<= 1) {
+        for (int p = t; p < dim / 2; p += 256) {
+            const int j = 2 * p - (p & (len - 1));
+            const float a = B[j], b = B[j + len];
+            B[j] = a + b;
+            B[j + len] = a - b;
+        }
+        __syncthreads();
+    }
+    // the rotated row (k_rotate's output) into A; with a TQ+ pair, k_calibrate's output over it
+    for (int i = t; i < dim; i += 256) A[i] = B[i] * inv_sqrt_block;
+    __syncthreads();
+    if (scale != nullptr) {
+        if (t == 0) {
+            double bc = 0.0;
+            for (int d = 0; d < dim; ++d) bc -= double(A[d]) * double(shift[d]);
+            s_bias = float(bc);
+        }
+        __syncthreads();
+        for (int i = t; i < dim; i += 256) A[i] = A[i] / scale[i];
+        __syncthreads();
+    }
+    const float *qc = A;
+    float m = 0.0f;
+    for (int d = t; d < dim; d += 256) m = fmaxf(m, fabsf(qc[d]));
+    const float qmax = block_max_256(m, red);
+    float qs = qmax / 127.0f, inv_qs;
+    if (qs >= FLT_MIN) inv_qs = 1.0f / qs; else { qs = 1.0f; inv_qs = 1.0f; }
+    for (int g = t; g < nch * 32; g += 256) {
+        int8_t lo = 0, hi = 0;
+        if (g < G) {
+            lo = int8_t(clamp_round_i8(qc[2 * g + 1] * inv_qs));
+            hi = int8_t(clamp_round_i8(qc[2 * g] * inv_qs));
+        }
+        base[wfrag_offset(g, n, 0, split)] = uint8_t(lo);
+        base[wfrag_offset(g, n, 1, split)] = uint8_t(hi);
+    }
+    if (t == 0) {
+        qscale[qi] = cs * qs;
+        qbias[qi] = 0.0f + (scale != nullptr ? s_bias : 0.0f);
+    }
+}
+
 // turbovec/src/search.rs:2856-2994 build_query_neon_lut_from_slice.  Output per
 // query: nch*32 rows of 32 bytes, row g = [16 entries indexed by the byte's HIGH
 // nibble (the group's first dimensions) | 16 entries indexed by the LOW nibble];
@@ -387,7 +472,9 @@ __device__ __forceinline__ void lds_settle_all(uint32_t (&e)[4], uint32_t (&o)[4
 template <int U, int MODE, bool W_LDS>
 __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
-    constexpr bool LISTS = MODE == kModeLists, DUMP = MODE == kModeDump, APPEND = MODE == kModeAppend;
+    constexpr bool LISTS = MODE == kModeLists, DUMP = MODE == kModeDump, BEST = MODE == kModeBest;
+    constexpr bool APPEND = MODE == kModeAppend || BEST;     // both fill the candidate segments
+    if (APPEND && launch_switched_off(a.run_if)) return;
     const int nch = a.nch, k = a.k;
     uint8_t *sW = smem + kDecodeBytes;
     const size_t w_bytes = kDecodeBytes + (W_LDS ? size_t(nch) * 2048 : 0);
@@ -418,7 +505,7 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
     const float qb = active ? a.qbias[qn] : 0.0f;
     const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
     // append mode: a fixed per-query floor; NaN for idle lanes so no compare passes
-    const float tau_fixed = APPEND ? (active ? order_unkey(a.gtau[qn]) : __int_as_float(0x7fc00000)) : 0.0f;
+    const float tau_fixed = (APPEND && !BEST) ? (active ? order_unkey(a.gtau[qn]) : __int_as_float(0x7fc00000)) : 0.0f;
 
     // Logical blocks j = 0..nj-1 stand for physical blocks j*step (step > 1 samples the index).
     const uint32_t step = a.b_step;
@@ -541,6 +628,28 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
                     }
                 }
             }
+        } else if (BEST) {
+            // A first sampling level without a floor: one candidate per block and query, the best
+            // allowed row of the block (a real score of a real row, so the k-th best of these is a
+            // floor at least k scanned rows reach, and with rows in no particular order it is the
+            // k-th best row of the sample but for the odd pair that shares a block).
+            float bs = 0.0f;
+            uint32_t bslot = 0xffffffffu;      // none yet
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = 8 * (r >> 2) + 4 * h + (r & 3);
+                const uint32_t slot = slot0 + i;
+                const float s = fmaf(float(acc[r]), qs, qb) * vs[r];
+                const bool ok = active && slot < a.n && ((mw >> i) & 1u) && s == s;
+                if (ok && (bslot == 0xffffffffu || ranks_before(s, slot, bs, bslot))) { bs = s; bslot = slot; }
+            }
+            const float os_ = __shfl_xor(bs, 32);
+            const uint32_t oslot = __shfl_xor(bslot, 32);
+            if (oslot != 0xffffffffu && (bslot == 0xffffffffu || ranks_before(os_, oslot, bs, bslot))) { bs = os_; bslot = oslot; }
+            if (h == 0 && bslot != 0xffffffffu) {
+                const uint32_t pos = atomicAdd(&scnt[qn], 1u);
+                if (pos < kSegCap) a.cand[(size_t(qn) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(bs, bslot);
+            }
         } else if (APPEND) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -601,6 +710,7 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
 template <int NT, int U, int THREADS>
 __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
+    if (launch_switched_off(a.run_if)) return;
     const int nch = a.nch;
     uint8_t *sW = smem + kDecodeBytes;                             // [NT][nch][2][64 lanes][16], after the byte table
     uint32_t *scnt = reinterpret_cast<uint32_t *>(sW + size_t(NT) * nch * 2048);
@@ -792,6 +902,7 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
 template <int NT, int MW, int KC, int OCC>
 __global__ __launch_bounds__(kScanThreads, OCC) void k_scan_p4_batched(ScanArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
+    if (launch_switched_off(a.run_if)) return;
     constexpr int kSliceBytes = NT * KC * 2048;           // one slice of all tiles
     constexpr int kStage = kSliceBytes / (kScanThreads * 16);  // uint4 per thread per slice
     static_assert(kSliceBytes % (kScanThreads * 16) == 0, "slice must split evenly over the workgroup");
@@ -1041,6 +1152,51 @@ __global__ __launch_bounds__(256) void k_merge(const float *__restrict__ part_sc
 // redo through the list path.
 // ===========================================================================
 
+// Largest value of v over the wave (all 64 lanes active), in every lane: four butterfly steps inside
+// each row of 16 lanes on the data-parallel path (no LDS), then the four row results through lane
+// reads.
+__device__ __forceinline__ uint32_t wave_umax(uint32_t v) {
+    v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0xB1, 0xf, 0xf, false)));    // quad_perm [1,0,3,2]
+    v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x4E, 0xf, 0xf, false)));    // quad_perm [2,3,0,1]
+    v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x141, 0xf, 0xf, false)));   // row_half_mirror
+    v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x140, 0xf, 0xf, false)));   // row_mirror
+    const uint32_t a = uint32_t(__builtin_amdgcn_readlane(int(v), 0)), b = uint32_t(__builtin_amdgcn_readlane(int(v), 16));
+    const uint32_t c = uint32_t(__builtin_amdgcn_readlane(int(v), 32)), d = uint32_t(__builtin_amdgcn_readlane(int(v), 48));
+    return max(max(a, b), max(c, d));
+}
+__device__ __forceinline__ uint64_t wave_umax64(uint64_t v) {
+    const uint32_t hi = uint32_t(v >> 32), lo = uint32_t(v);
+    const uint32_t mhi = wave_umax(hi);
+    const uint32_t mlo = wave_umax(hi == mhi ? lo : 0u);
+    return (uint64_t(mhi) << 32) | mlo;
+}
+// Eight keys in descending order (Batcher's odd-even merge network, 19 exchanges).
+__device__ __forceinline__ void sort8_desc(uint64_t (&r)[8]) {
+    auto ce = [&](int i, int j) { if (r[i] < r[j]) { const uint64_t x = r[i]; r[i] = r[j]; r[j] = x; } };
+    ce(0, 1); ce(2, 3); ce(4, 5); ce(6, 7);
+    ce(0, 2); ce(1, 3); ce(4, 6); ce(5, 7);
+    ce(1, 2); ce(5, 6);
+    ce(0, 4); ce(1, 5); ce(2, 6); ce(3, 7);
+    ce(2, 4); ce(3, 5);
+    ce(1, 2); ce(3, 4); ce(5, 6);
+}
+// The `need` (<= 32) largest of the wave's keys -- eight per lane, sorted descending, 0 = none,
+// non-zero keys distinct -- in order: lane i returns the i-th largest (0 beyond what there is).
+// One largest key is found and retired per turn; nothing touches LDS.
+__device__ __forceinline__ uint64_t wave_top(uint64_t (&r)[8], uint32_t need, uint32_t lane) {
+    uint64_t mine = 0ull;
+    for (uint32_t it = 0; it < need; ++it) {
+        const uint64_t m = wave_umax64(r[0]);
+        if (lane == it) mine = m;
+        if (r[0] == m && m != 0ull) {
+#pragma unroll
+            for (int e = 0; e < 7; ++e) r[e] = r[e + 1];
+            r[7] = 0ull;
+        }
+    }
+    return mine;
+}
+
 constexpr int kFinalThreads = 1024;
 constexpr int kFinalLong = kFinalCap / 8;   // segments of more than 8 keys that fit the sort buffer
 
@@ -1050,26 +1206,49 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
                                                float *__restrict__ out_scores, int64_t *__restrict__ out_idx,
                                                uint32_t *__restrict__ overflow, int *__restrict__ tau_out,
                                                int tau_stride_q, int keep_floor, int *__restrict__ raise_out,
-                                               const uint32_t *__restrict__ row_map) {
+                                               const uint32_t *__restrict__ row_map, uint32_t *level_over,
+                                               uint32_t *clear_flag, const uint32_t *run_if) {
     __shared__ uint64_t keys[kFinalCap];
     __shared__ uint32_t wave_sum[kFinalThreads / 64];
-    __shared__ uint32_t any_full, long_n;
+    __shared__ uint32_t any_full, long_n, any_long;
     __shared__ uint32_t long_seg[kFinalLong], long_pos[kFinalLong], long_cnt[kFinalLong];
     const int qn = blockIdx.x;
     const int t = threadIdx.x;
     const bool sampling = tau_out != nullptr;
     int *tau_slot = sampling ? tau_out + (qn / tau_stride_q) * kQTile + qn % tau_stride_q : nullptr;
-    if (t == 0) { any_full = 0u; long_n = 0u; }
+    if (launch_switched_off(run_if)) return;
+    if (clear_flag != nullptr && qn == 0 && t == 0) *clear_flag = 0u;
+    if (t == 0) { any_full = 0u; long_n = 0u; any_long = 0u; }
     __syncthreads();
     // every thread owns a contiguous run of this query's segments
     const uint32_t per = (n_seg + kFinalThreads - 1) / kFinalThreads;
     const uint32_t s0 = min(uint32_t(t) * per, n_seg), s1 = min(s0 + per, n_seg);
     const uint32_t *cnt = cand_cnt + size_t(qn) * seg_stride;
+    constexpr uint32_t kShort = 8;
+    // One segment per thread (the usual case): its head is requested together with its count, not
+    // after it -- the segment's memory is there whatever the count says -- which takes one trip to
+    // memory out of a kernel that is nothing but latency.
+    const bool one_each = per == 1;
+    uint64_t head[kShort];
+#pragma unroll
+    for (uint32_t e = 0; e < kShort; ++e) head[e] = 0ull;
     uint32_t mine = 0;
-    for (uint32_t sg = s0; sg < s1; ++sg) {
-        const uint32_t c = cnt[sg];
-        if (c > kSegCap) any_full = 1u;
-        mine += min(c, uint32_t(kSegCap));
+    if (one_each) {
+        if (s0 < s1) {
+            const uint64_t *src = cand + (size_t(qn) * seg_stride + s0) * kSegCap;
+            const uint32_t c = cnt[s0];
+#pragma unroll
+            for (uint32_t e = 0; e < kShort; ++e) head[e] = src[e];
+            if (c > kSegCap) any_full = 1u;
+            mine = min(c, uint32_t(kSegCap));
+            if (mine > kShort) any_long = 1u;
+        }
+    } else {
+        for (uint32_t sg = s0; sg < s1; ++sg) {
+            const uint32_t c = cnt[sg];
+            if (c > kSegCap) any_full = 1u;
+            mine += min(c, uint32_t(kSegCap));
+        }
     }
     // exclusive prefix over the 256 threads
     uint32_t incl = mine;
@@ -1082,6 +1261,10 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
     uint32_t base = incl - mine, total = 0;
     for (int w = 0; w < kFinalThreads / 64; ++w) { if (w < (t >> 6)) base += wave_sum[w]; total += wave_sum[w]; }
     const bool too_many = total > uint32_t(kFinalCap);
+    // A sampling level whose candidates did not all fit yields its floor from the subset that was
+    // kept: a valid floor, but possibly far below the k_floor-th best of the level.  The flag lets
+    // the caller's conditional launches repeat the level from that floor, which then fits.
+    if (sampling && level_over != nullptr && t == 0 && (too_many || any_full)) *level_over = 1u;
     // A final pass whose candidates did not fit: flag 1 = the caller repeats the full scan for this
     // query with the raised floor written below (the k_floor-th best of what was kept -- real
     // slots, so a valid lower bound of the true k-th best, and above the floor that let too many
@@ -1101,19 +1284,45 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
         if (t == 0 && !keep_floor) *tau_slot = kTauInit;
         return;
     }
+    const uint32_t c_all = min(total, uint32_t(kFinalCap));
+    const uint32_t need = (sampling || raising) ? min(uint32_t(k_floor), c_all) : uint32_t(k_eff);   // leading keys wanted, in order
+    // Few keys wanted and every thread already holds its whole segment in registers (the usual
+    // single-query case: some thousand candidates, a few per workgroup of the scan): no gather, no
+    // sort.  Every wave picks its `need` largest by rounds of wave-wide maxima, the 16 x 32 picks
+    // meet in LDS, and the first wave picks the `need` largest of those the same way.
+    const bool in_registers = one_each && any_long == 0u && need <= 32u;
+    if (in_registers) {
+        const uint32_t lane = uint32_t(t) & 63u, wv = uint32_t(t) >> 6;
+#pragma unroll
+        for (uint32_t e = 0; e < kShort; ++e) if (e >= mine) head[e] = 0ull;
+        sort8_desc(head);
+        const uint64_t pick = wave_top(head, need, lane);
+        if (lane < 32u) keys[wv * 32u + lane] = pick;
+        __syncthreads();
+        if (wv == 0) {
+            uint64_t r[8];
+#pragma unroll
+            for (uint32_t e = 0; e < 8; ++e) r[e] = keys[lane * 8u + e];
+            sort8_desc(r);
+            const uint64_t best = wave_top(r, need, lane);
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            if (lane < 32u) keys[lane] = best;
+        }
+        __syncthreads();
+    } else {
     // gather (a sampling level may keep any subset: dropping what does not fit only loosens the floor).
     // A thread copies a short segment itself, its loads in flight together; long ones (the first
     // sampling level fills a few segments to the brim) go on a list the waves then share, four
     // segments per wave and turn, a key per lane.
     uint32_t pos = base;
-    constexpr uint32_t kShort = 8;
     for (uint32_t sg = s0; sg < s1; ++sg) {
-        const uint32_t c = min(cnt[sg], uint32_t(kSegCap));
+        const uint32_t c = one_each ? mine : min(cnt[sg], uint32_t(kSegCap));
         const uint64_t *src = cand + (size_t(qn) * seg_stride + sg) * kSegCap;
         if (c <= kShort) {
             uint64_t v[kShort];
 #pragma unroll
-            for (uint32_t e = 0; e < kShort; ++e) v[e] = e < c ? src[e] : 0ull;
+            for (uint32_t e = 0; e < kShort; ++e) v[e] = one_each ? head[e] : (e < c ? src[e] : 0ull);
 #pragma unroll
             for (uint32_t e = 0; e < kShort; ++e)
                 if (e < c && pos + e < uint32_t(kFinalCap)) keys[pos + e] = v[e];
@@ -1153,8 +1362,6 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
         for (uint32_t u = 0; u < 4; ++u)
             if (ok[u]) keys[at[u]] = v[u];
     }
-    const uint32_t c_all = min(total, uint32_t(kFinalCap));
-    const uint32_t need = (sampling || raising) ? min(uint32_t(k_floor), c_all) : uint32_t(k_eff);   // leading keys wanted, in order
     uint32_t sort_n = need <= 64u ? 64u : 2u;
     while (sort_n < c_all) sort_n <<= 1;
     __syncthreads();
@@ -1220,6 +1427,7 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
             }
         }
     }
+    }   // gather and sort through LDS
     if (sampling || raising) {
         if (t == 0) {
             // the floor: the k_floor-th best sampled score (k_floor >= k_eff steadies the estimate)
@@ -1368,6 +1576,19 @@ hipError_t launch_build_p(const float *d_qcal, const float *d_bias_corr, uint8_t
     return hipGetLastError();
 }
 
+hipError_t launch_prep_p(const float *d_q, const float *d_signs, const uint32_t *d_perms, int dim, int block,
+                         float inv_sqrt_block, const float *d_shift, const float *d_scale, uint8_t *d_wfrag,
+                         float *d_qscale, float *d_qbias, int G, int nch, float cs, size_t nq, size_t nq_padded, bool split,
+                         hipStream_t s) {
+    if (nq_padded == 0) return hipSuccess;
+    const size_t lds = size_t(2) * dim * sizeof(float);
+    hipError_t e = allow_lds(k_prep_p, lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(k_prep_p, dim3(unsigned(nq_padded)), dim3(256), lds, s, d_q, d_signs, d_perms, dim, block,
+                       inv_sqrt_block, d_shift, d_scale, d_wfrag, d_qscale, d_qbias, G, nch, cs, nq, split);
+    return hipGetLastError();
+}
+
 hipError_t launch_build_lut(const float *d_qcal, const float *d_bias_corr, const float *d_centroids, uint8_t *d_lut,
                             float *d_qscale, float *d_qbias, int dim, int bits, int G, int nch, size_t nq,
                             size_t nq_padded, hipStream_t s) {
@@ -1411,7 +1632,7 @@ int scan_grid_blocks(int device, int mode_p, int nch, int k, int nq_tile) {
 
 hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s) {
     const size_t w = size_t(a.nch) * 2048;
-    const size_t lists = kDecodeBytes + (mode != kModeLists ? 64 : size_t(a.k) * kScanThreads * 8 + kQTile * sizeof(int));
+    const size_t lists = kDecodeBytes + kQTile * sizeof(int) + (mode != kModeLists ? 0 : size_t(a.k) * kScanThreads * 8);
     const bool w_lds = w + lists <= kLdsBudget;
     const size_t lds = (w_lds ? w : 0) + lists;
     hipError_t e = hipSuccess;
@@ -1425,6 +1646,7 @@ hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s) 
     do {                                                                                        \
         if (mode == kModeDump) { if (w_lds) TV_LAUNCH_P4(U, kModeDump, true); else TV_LAUNCH_P4(U, kModeDump, false); } \
         else if (mode == kModeAppend) { if (w_lds) TV_LAUNCH_P4(U, kModeAppend, true); else TV_LAUNCH_P4(U, kModeAppend, false); } \
+        else if (mode == kModeBest) { if (w_lds) TV_LAUNCH_P4(U, kModeBest, true); else TV_LAUNCH_P4(U, kModeBest, false); } \
         else { if (w_lds) TV_LAUNCH_P4(U, kModeLists, true); else TV_LAUNCH_P4(U, kModeLists, false); } \
     } while (0)
     if (a.nch % 8 == 0) TV_PICK_P4(8);          // 8 KiB per wave in flight: +3 % over 4 at 24 chunks, 12 is slower
@@ -1522,10 +1744,11 @@ hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, cons
 hipError_t launch_final(const uint64_t *cand, const uint32_t *cand_cnt, uint32_t n_seg, uint32_t seg_stride,
                         int k_eff, int k_floor, int nq, float *out_scores, int64_t *out_idx, uint32_t *overflow,
                         int *tau_out, int tau_stride_q, int keep_floor, int *raise_out, const uint32_t *row_map,
-                        hipStream_t s) {
+                        uint32_t *level_over, uint32_t *clear_flag, const uint32_t *run_if, hipStream_t s) {
     if (nq == 0 || k_eff == 0) return hipSuccess;
     hipLaunchKernelGGL(k_final, dim3(nq), dim3(kFinalThreads), 0, s, cand, cand_cnt, n_seg, seg_stride, k_eff, k_floor,
-                       out_scores, out_idx, overflow, tau_out, tau_stride_q, keep_floor, raise_out, row_map);
+                       out_scores, out_idx, overflow, tau_out, tau_stride_q, keep_floor, raise_out, row_map, level_over,
+                       clear_flag, run_if);
     return hipGetLastError();
 }
 

@@ -100,6 +100,7 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
     typedef typename LutWord<QL>::type word_t;
     constexpr bool LISTS = MODE == kModeLists, DUMP = MODE == kModeDump, APPEND = MODE == kModeAppend;
     extern __shared__ __align__(16) uint8_t smem[];
+    if (APPEND && launch_switched_off(a.run_if)) return;
     const int nch = a.nch, k = a.k;
     const size_t lut_bytes = LUT_LDS ? size_t(nch) * 1024 * QL : 0;
     float *sct = reinterpret_cast<float *>(smem + lut_bytes);            // [waves][QL][32]
@@ -386,6 +387,7 @@ constexpr int kLutBtThreads = 1024;
 template <int U>
 __global__ __launch_bounds__(kLutBtThreads) void k_scan_lut_bt(ScanArgs a, int n_bt) {
     extern __shared__ __align__(16) uint8_t smem[];
+    if (launch_switched_off(a.run_if)) return;
     const int nch = a.nch;
     uint8_t *bt = smem;                                                   // [n_bt * 32][256]
     uint8_t *nt = smem + size_t(n_bt) * 8192;                             // [(nch - n_bt) * 32][32]: the nibble tables as built

@@ -110,6 +110,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     static_assert(KS == 1 || (KS == 2 && WAVES == 4 && BLK == 1 && HO == 1), "row halves go to the wave pairs of the four-wave form");
     static_assert(HO == 1 || (SPT % HO == 0 && kWideRing >= 2 * HO + 1), "slices handed over together must fit the ring twice");
     extern __shared__ __align__(16) uint8_t smem[];
+    if (launch_switched_off(a.run_if)) return;
     constexpr int kWideThreads = WAVES * 64, kWideWaves = WAVES;
     constexpr int kSC = NCH / SPT;                          // chunks per slice
     constexpr int kM = 2 * kSC;                             // MFMAs per wave and slice: (low, high) of each chunk
