@@ -154,8 +154,11 @@ int tv_search_dev(tv_index *ix, const float *d_queries, size_t nq, size_t k,
                   const uint64_t *d_mask_words, size_t n_allowed,
                   float *d_out_scores, int64_t *d_out_indices, size_t *out_k_eff);
 
-/* tv_search_dev for callers that cannot allocate device memory (code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+/* tv_search_dev for callers that cannot allocate device memory (tight serving loops, harnesses
+ * that forbid hipMalloc, code that must not disturb a caching allocator).  No counterpart in the
+ * reference.  Like tv_search_dev it runs on the index's own stream and synchronises that stream
+ * before it returns (it reads the overflow flags of its passes on the host), so it cannot be
+ * recorded into a HIP graph under capture.
  * Same arguments, results and status codes as tv_search_dev, but everything the search carves
  * -- rotated queries, tables, candidate segments, the exact path's lists -- comes out of a
  * fixed array in the library's device image (tv_noalloc_scratch_bytes() bytes, 64 MiB, held by
@@ -245,6 +248,9 @@ int tv_debug_sampling_plan(const tv_index *ix, size_t nq, size_t k, uint32_t *st
  * makes searches report such levels (a few hundred bytes more in the flag copy), 0 stops that,
  * negative leaves it as it is; *count (may be NULL) = levels repeated so far while tracking. */
 int tv_debug_level_repeats(tv_index *ix, int track, size_t *count);
+/* Bytes of the index's cached search workspace and of its host-call staging allocation (either
+ * pointer may be NULL): both only ever grow, and tv_search_dev_noalloc touches neither. */
+int tv_debug_workspace_bytes(const tv_index *ix, size_t *workspace, size_t *staging);
 /* How many queries so far did not finish in the single sampled pass because their
  * candidate buffer overflowed (they are scanned once more, all together, from a raised
  * floor), and how many of those went on to the exact list / select path. */

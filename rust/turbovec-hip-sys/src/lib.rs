@@ -89,6 +89,7 @@ extern "C" {
     pub fn tv_debug_set_path(ix: *mut tv_index, force_full_lists: c_int) -> c_int;
     pub fn tv_debug_sampling_plan(ix: *const tv_index, nq: usize, k: usize, strides: *mut u32, repeat_offsets: *mut u32, cap: usize, count: *mut usize) -> c_int;
     pub fn tv_debug_level_repeats(ix: *mut tv_index, track: c_int, count: *mut usize) -> c_int;
+    pub fn tv_debug_workspace_bytes(ix: *const tv_index, workspace: *mut usize, staging: *mut usize) -> c_int;
     pub fn tv_debug_overflow_redos(ix: *const tv_index, count: *mut usize) -> c_int;
     pub fn tv_debug_exact_redos(ix: *const tv_index, count: *mut usize) -> c_int;
     pub fn tv_debug_merged_calls(ix: *const tv_index, count: *mut usize) -> c_int;

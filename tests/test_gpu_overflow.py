@@ -101,6 +101,21 @@ def test_merged_calls_return_each_callers_rows(T, oracle, dev_buffers):
     words = T.pack_mask(mask)[0]
     want_masked = [oidx.search(q, k, mask_words=words) for q in qs]
     bad = []
+    dev_bufs = []
+    if dev_buffers:                      # device buffers are made on this thread, before the callers start
+        dev = torch.device("cuda:0")
+        for q in qs:
+            dev_bufs.append((torch.from_numpy(q).to(dev), torch.empty(len(q), k, device=dev),
+                             torch.empty(len(q), k, dtype=torch.int64, device=dev)))
+        torch.cuda.synchronize()
+
+    def guarded(fn):
+        def run(t):
+            try:
+                fn(t)
+            except Exception as e:       # a thread's exception must fail the test, not vanish
+                bad.append((t, repr(e)))
+        return run
 
     def host_worker(t):
         for it in range(per_thread):
@@ -111,17 +126,14 @@ def test_merged_calls_return_each_callers_rows(T, oracle, dev_buffers):
                 bad.append((t, it))
 
     def dev_worker(t):
-        dev = torch.device("cuda:0")
-        dq = torch.from_numpy(qs[t]).to(dev)
-        ds = torch.empty(len(qs[t]), k, device=dev)
-        di = torch.empty(len(qs[t]), k, dtype=torch.int64, device=dev)
-        torch.cuda.synchronize()
+        dq, ds, di = dev_bufs[t]
         for it in range(per_thread):
             ix.search_dev(dq.data_ptr(), len(qs[t]), k, ds.data_ptr(), di.data_ptr())
             if not (np.array_equal(di.cpu().numpy(), want[t][1]) and bits_equal(ds.cpu().numpy(), want[t][0])):
                 bad.append((t, it))
 
-    threads = [threading.Thread(target=dev_worker if dev_buffers else host_worker, args=(t,)) for t in range(n_threads)]
+    threads = [threading.Thread(target=guarded(dev_worker if dev_buffers else host_worker), args=(t,))
+               for t in range(n_threads)]
     for th in threads:
         th.start()
     for th in threads:

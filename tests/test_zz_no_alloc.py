@@ -106,3 +106,24 @@ def test_noalloc_refuses_what_does_not_fit(T):
     assert ix.search_dev_noalloc(q.data_ptr(), 4, 0, s.data_ptr(), i.data_ptr()) == 0
     assert ix.search_dev_noalloc(q.data_ptr(), 0, 10, s.data_ptr(), i.data_ptr()) == 10
     ix.close()
+
+
+def test_noalloc_takes_no_device_memory(T):
+    """Free device memory and the index's own workspace stay what they were across calls of the
+    entry point, on an index whose regular workspace was never sized for these searches."""
+    ix, gen = build(T, 120_000, 256, 4, seed=13)
+    dev = torch.device("cuda:0")
+    q = torch.randn(96, 256, device=dev, generator=gen)
+    s = torch.zeros(96, 10, device=dev)
+    i = torch.zeros(96, 10, dtype=torch.int64, device=dev)
+    torch.cuda.synchronize()
+    ws0 = ix.workspace_bytes()
+    free0 = torch.cuda.mem_get_info()[0]
+    for nq in (96, 40, 1, 96):
+        ix.search_dev_noalloc(q.data_ptr(), nq, 10, s.data_ptr(), i.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    assert ix.workspace_bytes() == ws0
+    ix.search_dev(q.data_ptr(), 96, 10, s.data_ptr(), i.data_ptr())      # the regular entry point does grow it
+    assert ix.workspace_bytes()[0] > ws0[0]
+    ix.close()

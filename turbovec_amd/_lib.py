@@ -33,7 +33,7 @@ EXPORTS = [
     "tv_debug_stream_probe", "tv_debug_mfma_probe", "tv_debug_set_path", "tv_debug_overflow_redos",
     "tv_host_snapshot_len", "tv_host_snapshot_compose", "tv_host_snapshot_info", "tv_host_snapshot_extract",
     "tv_index_to_bytes", "tv_index_from_bytes", "tv_search_dev_noalloc", "tv_noalloc_scratch_bytes",
-    "tv_debug_exact_redos", "tv_debug_sampling_plan", "tv_debug_merged_calls", "tv_debug_level_repeats",
+    "tv_debug_exact_redos", "tv_debug_sampling_plan", "tv_debug_merged_calls", "tv_debug_level_repeats", "tv_debug_workspace_bytes",
 ]
 
 _lib = None
@@ -100,6 +100,7 @@ def lib():
     L.tv_debug_set_path.argtypes = [vp, i32]
     L.tv_debug_overflow_redos.argtypes = [vp, C.POINTER(sz)]
     L.tv_debug_exact_redos.argtypes = [vp, C.POINTER(sz)]
+    L.tv_debug_workspace_bytes.argtypes = [vp, C.POINTER(sz), C.POINTER(sz)]
     L.tv_debug_level_repeats.argtypes = [vp, i32, C.POINTER(sz)]
     L.tv_debug_merged_calls.argtypes = [vp, C.POINTER(sz)]
     L.tv_debug_sampling_plan.argtypes = [vp, sz, sz, vp, vp, sz, C.POINTER(sz)]
@@ -313,6 +314,12 @@ class NativeIndex:
         c = C.c_size_t(0)
         check(lib().tv_debug_exact_redos(self.h, C.byref(c)))
         return c.value
+
+    def workspace_bytes(self):
+        """(search workspace, host-call staging) bytes the index holds on the device."""
+        a, b = C.c_size_t(0), C.c_size_t(0)
+        check(lib().tv_debug_workspace_bytes(self.h, C.byref(a), C.byref(b)))
+        return a.value, b.value
 
     def level_repeats(self, track=-1):
         """Sampling levels that ran twice so far (counted while tracking is on; track=1/0 switches it)."""

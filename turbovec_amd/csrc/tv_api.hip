@@ -870,7 +870,7 @@ bool compatible(const tv_request &a, const tv_request &b) {
 // How long a caller that is about to serve waits for the callers of the batch before to come back
 // with their next call (they were all released at the same moment and are a few microseconds of
 // host code away from asking again).  Only after a batch that did merge calls.
-constexpr auto kGatherWait = std::chrono::microseconds(150);
+constexpr auto kGatherWait = std::chrono::microseconds(300);
 
 int search_merged(tv_index *ix, tv_request &r) {
     std::vector<tv_request *> batch;
@@ -974,7 +974,9 @@ int tv_index_create(int dim, int bits, int device, tv_index **out) {
     // 4-bit rows are padded with whole chunks of zero groups (their query weights are zero, so they
     // add nothing) up to a chunk count the all-queries-per-pass kernel has an instance for: even
     // from 9 chunks on, a multiple of 4 above 24, of 8 above 48 (to 96 chunks = 6144 dimensions).
-    // At most one chunk in nine of extra code bytes.
+    // The padding is part of the resident index on every path: at most 3 chunks (of 25: +12 %), 7
+    // (of 49: +14 %), one in seven at worst; the device block is geo.block_bytes() = nch * 1024
+    // bytes, not ceil(G / 32) * 1024.
     if (bits == 4 && ix->geo.nch >= 9) {
         if (ix->geo.nch > 48 && ix->geo.nch <= 96) ix->geo.nch = (ix->geo.nch + 7) / 8 * 8;
         else if (ix->geo.nch > 24 && ix->geo.nch <= 48) ix->geo.nch = (ix->geo.nch + 3) / 4 * 4;
@@ -1674,6 +1676,15 @@ int tv_debug_level_repeats(tv_index *ix, int track, size_t *count) {
     std::lock_guard<std::mutex> lock(ix->mu);
     if (track >= 0) ix->track_levels = track;
     if (count) *count = ix->level_repeats;
+    return TV_OK;
+}
+
+int tv_debug_workspace_bytes(const tv_index *cix, size_t *workspace, size_t *staging) {
+    tv_index *ix = const_cast<tv_index *>(cix);
+    if (!ix) return TV_ERR_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(ix->mu);
+    if (workspace) *workspace = ix->ws_bytes;
+    if (staging) *staging = ix->io_bytes;
     return TV_OK;
 }
 

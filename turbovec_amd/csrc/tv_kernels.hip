@@ -469,6 +469,27 @@ __device__ __forceinline__ void lds_settle_all(uint32_t (&e)[4], uint32_t (&o)[4
     for (int t = 0; t < NT; ++t) asm volatile("" : "+v"(w[t]));
 }
 
+// n16 16-byte words from global memory into LDS by a workgroup of THREADS, twelve loads per thread
+// in flight at a time: a scan launch that reads a block or two per wave (a sampling level, a
+// small index) is as long as its set-up, and word after word the copy is a chain of trips to L2.
+template <int THREADS>
+__device__ __forceinline__ void stage_to_lds(uint4 *dst, const uint4 *src, int n16, int tid) {
+    constexpr int kBatch = 12;
+    for (int i0 = tid; i0 < n16; i0 += THREADS * kBatch) {
+        uint4 tmp[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const int i = i0 + u * THREADS;
+            tmp[u] = i < n16 ? src[i] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const int i = i0 + u * THREADS;
+            if (i < n16) dst[i] = tmp[u];
+        }
+    }
+}
+
 template <int U, int MODE, bool W_LDS>
 __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
@@ -484,28 +505,8 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
     uint32_t *scnt = reinterpret_cast<uint32_t *>(stau);  // append mode: candidates per query of this workgroup
 
     const int tid = threadIdx.x;
-    if (W_LDS) {
-        const uint4 *src = reinterpret_cast<const uint4 *>(a.tables);
-        uint4 *dst = reinterpret_cast<uint4 *>(sW);
-        for (int i = tid; i < nch * 128; i += kScanThreads) dst[i] = src[i];
-    }
-    for (int b = tid; b < 256; b += kScanThreads) {
-        const uint32_t lo = (a.lv[(b & 15) >> 2] >> (8 * (b & 3))) & 0xffu;
-        const uint32_t hi = (a.lv[b >> 6] >> (8 * ((b >> 4) & 3))) & 0xffu;
-        reinterpret_cast<uint16_t *>(smem)[b] = uint16_t(lo | (hi << 8));
-    }
-    if (LISTS && tid < kQTile) stau[tid] = a.gtau[tid];
-    if (APPEND && tid < kQTile) scnt[tid] = 0u;
-    __syncthreads();
-
     const int lane = tid & 63, wave = tid >> 6;
     const int qn = lane & 31, h = lane >> 5;
-    const bool active = qn < a.nq_tile;
-    const float qs = active ? a.qscale[qn] : 0.0f;
-    const float qb = active ? a.qbias[qn] : 0.0f;
-    const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
-    // append mode: a fixed per-query floor; NaN for idle lanes so no compare passes
-    const float tau_fixed = (APPEND && !BEST) ? (active ? order_unkey(a.gtau[qn]) : __int_as_float(0x7fc00000)) : 0.0f;
 
     // Logical blocks j = 0..nj-1 stand for physical blocks j*step (step > 1 samples the index).
     const uint32_t step = a.b_step;
@@ -516,11 +517,7 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
     // gw + total_waves, ...  Neighbouring rows (clustered data, contiguous allowlists) then spread
     // over all workgroups instead of piling into one.
     const uint32_t j_begin = gw, j_end = nj;
-
-    LaneList L{0, 0.0f, 0u, 0};
     const uint4 *codes = reinterpret_cast<const uint4 *>(a.codes) + lane;
-    const uint4 *wglob = reinterpret_cast<const uint4 *>(a.tables) + lane;
-    const uint4 *wlds = reinterpret_cast<const uint4 *>(sW) + lane;
 
     // first block with at least one allowed slot (search.rs:3015-3029)
     auto live_from = [&](uint32_t j) -> uint32_t {
@@ -534,12 +531,34 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
         return j;
     };
 
+    // the wave's first codes are on their way from HBM while the workgroup sets up its LDS
     uint32_t j = live_from(j_begin);
     uint4 buf[U];
     if (j < j_end) {
 #pragma unroll
         for (int u = 0; u < U; ++u) buf[u] = load_stream16(&codes[(size_t(j) * step * nch + u) * 64]);
     }
+
+    if (W_LDS) stage_to_lds<kScanThreads>(reinterpret_cast<uint4 *>(sW), reinterpret_cast<const uint4 *>(a.tables), nch * 128, tid);
+    for (int b = tid; b < 256; b += kScanThreads) {
+        const uint32_t lo = (a.lv[(b & 15) >> 2] >> (8 * (b & 3))) & 0xffu;
+        const uint32_t hi = (a.lv[b >> 6] >> (8 * ((b >> 4) & 3))) & 0xffu;
+        reinterpret_cast<uint16_t *>(smem)[b] = uint16_t(lo | (hi << 8));
+    }
+    if (LISTS && tid < kQTile) stau[tid] = a.gtau[tid];
+    if (APPEND && tid < kQTile) scnt[tid] = 0u;
+    __syncthreads();
+
+    const bool active = qn < a.nq_tile;
+    const float qs = active ? a.qscale[qn] : 0.0f;
+    const float qb = active ? a.qbias[qn] : 0.0f;
+    const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
+    // append mode: a fixed per-query floor; NaN for idle lanes so no compare passes
+    const float tau_fixed = (APPEND && !BEST) ? (active ? order_unkey(a.gtau[qn]) : __int_as_float(0x7fc00000)) : 0.0f;
+
+    LaneList L{0, 0.0f, 0u, 0};
+    const uint4 *wglob = reinterpret_cast<const uint4 *>(a.tables) + lane;
+
     while (j < j_end) {
         const uint32_t nj_live = live_from(j + total_waves);
         const uint32_t b = j * step;
@@ -718,10 +737,9 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
     const int qn = lane & 31, h = lane >> 5;
     const int nt_active = (a.nq_tile + kQTile - 1) / kQTile;
     {
-        const uint4 *src = reinterpret_cast<const uint4 *>(a.tables);
-        uint4 *dst = reinterpret_cast<uint4 *>(sW);
         const int live16 = nt_active * nch * 128;
-        for (int i = tid; i < NT * nch * 128; i += THREADS) dst[i] = i < live16 ? src[i] : make_uint4(0, 0, 0, 0);
+        stage_to_lds<THREADS>(reinterpret_cast<uint4 *>(sW), reinterpret_cast<const uint4 *>(a.tables), live16, tid);
+        for (int i = live16 + tid; i < NT * nch * 128; i += THREADS) reinterpret_cast<uint4 *>(sW)[i] = make_uint4(0, 0, 0, 0);
     }
     for (int b = tid; b < 256; b += THREADS) {   // code byte -> (level of its low nibble, level of its high nibble)
         const uint32_t lo = (a.lv[(b & 15) >> 2] >> (8 * (b & 3))) & 0xffu;
@@ -1706,7 +1724,11 @@ static hipError_t launch_multi_u(const ScanArgs &a, int grid, hipStream_t s) {
 
 template <int NT>
 static hipError_t launch_multi(const ScanArgs &a, int grid, hipStream_t s) {
-    if (a.nch % 4 == 0) return launch_multi_u<NT, 4>(a, grid, s);
+    // (four tiles' accumulators and four-chunk bursts together do not fit the 168 registers three
+    // waves per SIMD leave: the compiler would spill, which the hand-placed waits cannot allow)
+    if constexpr (NT < 4) {
+        if (a.nch % 4 == 0) return launch_multi_u<NT, 4>(a, grid, s);
+    }
     if (a.nch % 2 == 0) return launch_multi_u<NT, 2>(a, grid, s);
     return launch_multi_u<NT, 1>(a, grid, s);
 }

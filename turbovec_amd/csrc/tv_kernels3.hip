@@ -304,6 +304,10 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
         // workgroup could still append would be kept, so it claims no further blocks.  (A floor
         // far too low -- rows arranged against the sampler -- ends the launch within a few rounds
         // instead of scoring the whole index for nothing.)
+        // (The two waves of a pair must see the same value -- one claiming a block while its partner
+        // sits out would add stale partial sums -- so the pair form reads it behind a barrier every
+        // wave's appends of the round before have passed.)
+        if constexpr (KS == 2) __syncthreads();
         const bool futile = uint32_t(__builtin_amdgcn_readfirstlane(int(*reinterpret_cast<volatile uint32_t *>(s_over)))) >= uint32_t(nq);
         static_for<BLK>([&](auto kk) {
             constexpr int k = decltype(kk)::value;
@@ -532,8 +536,8 @@ int wide_blocks_per_workgroup(int nch) {
         case 2: return 48;
         case 4: return 32;
         case 6: return 24;
-        case 8: case 10: case 12: return 16;
-        case 14: case 16: case 18: case 20: case 22: case 24: return 8;
+        case 8: case 10: return 16;
+        case 12: case 14: case 16: case 18: case 20: case 22: case 24: return 8;
         case 28: case 32: case 36: case 40: case 44: case 48: return 4;
         case 56: case 64: case 72: case 80: case 88: case 96: return 2;
         default: return 0;
@@ -579,7 +583,7 @@ hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s) {
         case 6: return launch_wide_n<6, 2, 8, 1, 3>(a, grid, s);
         case 8: return launch_wide_n<8, 4, 8, 1, 2>(a, grid, s);
         case 10: return launch_wide_n<10, 2, 8, 2, 2, 2>(a, grid, s);
-        case 12: return launch_wide_n<12, 2, 8, 2, 2, 2>(a, grid, s);
+        case 12: return launch_wide_n<12, 2, 8, 2, 1, 2>(a, grid, s);   // two blocks per wave would spill 21 registers
         case 14: return launch_wide_n<14, 2, 8, 2, 1, 2>(a, grid, s);
         case 16: return launch_wide_n<16, 4, 8, 2, 1, 2>(a, grid, s);
         case 18: return launch_wide_n<18, 2, 8, 2, 1, 2>(a, grid, s);
