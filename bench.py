@@ -226,7 +226,10 @@ def adversarial_extra(T, torch, run, args, normal_ms, ladder):
     u = u / u.norm()
     q = u + 0.5 * torch.randn(nq, dim, device=dev, generator=gen) / dim ** 0.5
     q = (q / q.norm(dim=1, keepdim=True)).contiguous()
-    for key, poisoned in (("every_sampling_level_poisoned", strides[:-1]), ("first_sampling_level_poisoned", strides[:1])):
+    layouts = [("every_sampling_level_poisoned", strides[:-1])]
+    if len(strides) > 2:      # with one sampling level only, the two layouts are the same
+        layouts.append(("first_sampling_level_poisoned", strides[:1]))
+    for key, poisoned in layouts:
         ix = T.NativeIndex(dim, 4)
         for c0 in range(0, n, 100_000):
             blocks = torch.arange(c0, c0 + 100_000, device=dev) // 32

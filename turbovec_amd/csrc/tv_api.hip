@@ -481,14 +481,23 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
 // 8 * k_floor blocks; a quarter of the index or more is not worth sampling.
 constexpr size_t kBestLevelMaxK = 64;
 bool first_level_is_best_of_block(const tv_index *ix, const SampledPlan &plan, size_t k_floor) {
-    return effective_mode(ix) == TV_SCORE_P && !plan.wide && plan.nt_batched == 0 && k_floor <= kBestLevelMaxK;
+    return effective_mode(ix) == TV_SCORE_P && k_floor <= kBestLevelMaxK &&
+           (plan.wide ? tv::wide_serves_best_of_block(ix->geo.nch) : plan.nt_batched == 0);
 }
 SamplingSteps level_strides(const tv_index *ix, const SampledPlan &plan, size_t n_blocks, size_t k_floor, bool repeat) {
     if (!repeat && first_level_is_best_of_block(ix, plan, k_floor)) {
         SamplingSteps steps;
         size_t sample = std::max<size_t>((n_blocks * k_floor + 2047) / 2048, 8 * k_floor);
         sample = std::min<size_t>(sample, size_t(plan.grid) * (tv::kSegCap / 2));   // a workgroup's blocks fit its segment
-        if (sample * 4 <= n_blocks && n_blocks / sample > 1) steps.step[steps.count++] = uint32_t(n_blocks / sample);
+        size_t step = sample ? n_blocks / sample : 0;
+        if (plan.wide) {
+            // the all-queries-per-pass kernel works through the blocks in rounds of its grid and a
+            // level costs whole rounds: trimmed to whole rounds, at least one, and never spilling into another
+            const size_t round = size_t(plan.grid) * tv::wide_blocks_per_workgroup(ix->geo.nch);
+            if (sample > round) sample -= sample % round;
+            step = sample >= round ? (n_blocks + sample - 1) / sample : n_blocks / sample;
+        }
+        if (sample * 4 <= n_blocks && step > 1) steps.step[steps.count++] = uint32_t(step);
         steps.step[steps.count++] = 1;
         return steps;
     }
@@ -625,6 +634,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
                         a.gtau = ((lv == 0 && !repeat) ? ix->d_tau_open : d_tau) + t * tv::kQTile;
                         a.b_step = steps[lv];
                         a.run_if = run_if;
+                        a.best_of_block = (best_first && lv == 0) ? 1 : 0;
                         if (off) {
                             a.codes += size_t(off) * g.block_bytes();
                             a.scales += size_t(off) * tv::kVecBlock;

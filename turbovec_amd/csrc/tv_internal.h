@@ -67,6 +67,7 @@ struct ScanArgs {
     uint64_t *cand;            // append mode: [nq_tile][seg_stride][kSegCap] sort keys, one segment per workgroup
     uint32_t *cand_cnt;        // append mode: [nq_tile][seg_stride] counts (above kSegCap: that segment overflowed)
     uint32_t seg_stride;       // segments allocated per query (>= grid of the launch)
+    int best_of_block;         // all-queries-per-pass kernel: no floor, per scanned block and query the best allowed slot (kModeBest)
     const uint32_t *run_if;    // append mode: when given and *run_if == 0 the launch does nothing (a level's conditional repeat)
 };
 
@@ -124,6 +125,7 @@ int wide_min_queries(int nch);
 int wide_grid_blocks(int device);
 hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s);
 int wide_blocks_per_workgroup(int nch);
+bool wide_serves_best_of_block(int nch);
 
 hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, const int *part_cnt, int total_threads,
                         int qmod, int k, int k_eff, int nq_tile, float *out_scores, int64_t *out_idx,

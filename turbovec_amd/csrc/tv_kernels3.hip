@@ -396,6 +396,33 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
                 }
             }
         };
+        // A first sampling level without floors (a.best_of_block): per tile and block the lane's best
+        // allowed row, the better of the two lanes that share a query, one candidate per block and
+        // query -- a real score of a real row, so the k-th best of these is a floor k scanned rows
+        // reach.  One launch over a round of blocks; the hot loop never comes here.
+        auto best_tile = [&](int q, auto kk) {
+            constexpr int k = decltype(kk)::value;
+            const float4 qp = *reinterpret_cast<const float4 *>(&sq[q].qs);
+            const float qs = qp.x, qb = qp.y;
+            const float *vs = s_vs + (wave * BLK + k) * 32 + 4 * h;
+            float bs = 0.0f;
+            int bi = -1;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = 8 * (r >> 2) + (r & 3);
+                const float s = fmaf(float(acc[k][r]), qs, qb) * vs[i];
+                if (s == s && (bi < 0 || s > bs)) { bs = s; bi = i + 4 * h; }    // rows in rising order: ties keep the lower slot
+            }
+            const float os_ = __shfl_xor(bs, 32);
+            const int oi = __shfl_xor(bi, 32);
+            if (oi >= 0 && (bi < 0 || os_ > bs || (os_ == bs && oi < bi))) { bs = os_; bi = oi; }
+            if (h == 0 && bi >= 0 && q < nq) {
+                const uint32_t pos = atomicAdd(&sq[q].cnt, 1u);
+                if (pos < kSegCap)
+                    a.cand[(size_t(q) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(bs, blk[k] * 32u + uint32_t(bi));
+            }
+        };
+        const bool best_mode = BLK == 1 && a.best_of_block != 0;   // (several blocks per wave: no registers to spare for it)
         if (has) open_stream();
         for (int t = 0; t < nt; ++t) {
             const int q = t * kQTile + qn;
@@ -435,6 +462,9 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
                 if (KS == 1 || part == 0) static_for<BLK>([&](auto kk) {
                     constexpr int k = decltype(kk)::value;
                     if constexpr (kHandMfma && KS == 1) mfma_settle(acc[k]);
+                    if constexpr (BLK == 1) {
+                        if (best_mode) { best_tile(q, kk); return; }
+                    }
                     const v16i &c = acc[k];
                     int m0 = max(max(c[0], c[1]), c[2]), m1 = max(max(c[3], c[4]), c[5]);
                     int m2 = max(max(c[6], c[7]), c[8]), m3 = max(max(c[9], c[10]), c[11]);
@@ -528,6 +558,9 @@ int wide_min_queries(int nch) {
         default: return 0;
     }
 }
+
+// Whether the instance for this row length serves a first level without floors (ScanArgs::best_of_block).
+bool wide_serves_best_of_block(int nch) { return nch >= 12 && wide_blocks_per_workgroup(nch) > 0; }
 
 // Blocks one workgroup of the instance for this row length holds per round (waves x blocks per
 // wave, or wave pairs); 0 = no instance.
