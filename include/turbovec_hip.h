@@ -59,6 +59,8 @@ typedef enum {
  * time from CPU features, turbovec/src/pack.rs:1189-1219, search.rs:2975-2980). */
 typedef enum {
     TV_SCORE_AUTO = 0,      /* what an AVX-512 VNNI / dotprod host runs: P at 4-bit, L_U32 at 2/3-bit */
+    TV_SCORE_L_SCALAR = 1,  /* u8 LUT terms added one by one in f32, bias first   search.rs:3113-3128 (the
+                               definition; what FORCE_SCALAR_FALLBACK selects, search.rs:313-316) */
     TV_SCORE_L_CLASSIC = 2, /* u8 LUT sums, fma flush per 256 byte-groups   search.rs:516-582 */
     TV_SCORE_L_U32 = 3,     /* u8 LUT sums, (acc*scale+bias)*vec_scale      search.rs:1174-1177 */
     TV_SCORE_P = 4          /* int8 permute-dot, fma(acc,scale,bias)*vs     search.rs:1519-1524 (4-bit only) */

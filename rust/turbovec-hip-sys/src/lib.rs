@@ -33,6 +33,7 @@ pub const TV_ERR_BAD_IMAGE: c_int = 10;
 
 // tv_score_mode
 pub const TV_SCORE_AUTO: c_int = 0;
+pub const TV_SCORE_L_SCALAR: c_int = 1;
 pub const TV_SCORE_L_CLASSIC: c_int = 2;
 pub const TV_SCORE_L_U32: c_int = 3;
 pub const TV_SCORE_P: c_int = 4;

@@ -47,6 +47,10 @@ CASES = [
     (1536, 2, 3000, 2, 10, "L_CLASSIC"),
     (64, 3, 1500, 3, 10, "L_U32"),
     (1000, 2, 2000, 3, 5, "L_U32"),        # B = 8 rotation blocks
+    (128, 4, 3000, 7, 10, "L_SCALAR"),     # the definition: every LUT term added in f32, one by one
+    (1536, 2, 3000, 3, 10, "L_SCALAR"),
+    (200, 4, 3000, 4, 7, "L_SCALAR"),      # padded last chunk: the chain stops at the last real group
+    (64, 3, 1500, 3, 100, "L_SCALAR"),     # k beyond the per-lane lists
     (128, 4, 3000, 3, 100, "P"),           # k beyond the per-lane lists: radix select
     (64, 3, 500, 3, 500, "L_U32"),         # k = n: full ranking
     (128, 2, 5000, 2, 1000, "L_U32"),
@@ -180,7 +184,7 @@ def test_config1_full(T, oracle):
 
 
 # ---- filtering: turbovec/tests/filtering.rs ----
-@pytest.mark.parametrize("bits,mode", [(4, "P"), (2, "L_U32"), (4, "L_CLASSIC")])
+@pytest.mark.parametrize("bits,mode", [(4, "P"), (2, "L_U32"), (4, "L_CLASSIC"), (2, "L_SCALAR")])
 def test_mask_semantics(T, oracle, bits, mode):
     O = oracle
     dim, n, nq = 128, 4000, 6
@@ -285,7 +289,7 @@ def test_tqplus_calibration(T, oracle):
     cal = O.fit_calibration(rot, v, cen)
     oidx = OracleIndex(O, dim, bits, v, calibration=cal)
     q = O.lcg_vectors(6, dim, 77)
-    for mode in ("P", "L_CLASSIC"):
+    for mode in ("P", "L_CLASSIC", "L_SCALAR"):
         ix = to_native(T, oidx, tmode(T, mode))
         s, i = ix.search(q, 10)
         os_, oi = oidx.search(q, 10, mode=omode(O, mode))
@@ -446,7 +450,7 @@ def test_random_codes_scale_properties(T):
 
 
 # ---- sample-then-filter path (n above the candidate capacity) ----
-@pytest.mark.parametrize("bits,mode", [(4, "P"), (2, "L_U32"), (4, "L_CLASSIC")])
+@pytest.mark.parametrize("bits,mode", [(4, "P"), (2, "L_U32"), (4, "L_CLASSIC"), (4, "L_SCALAR")])
 def test_sampled_path_matches_oracle_and_full_path(T, oracle, bits, mode):
     O = oracle
     dim, n, nq = 128, 40_003, 37

@@ -21,7 +21,7 @@ ERR_HIP = 7
 ERR_NO_DEVICE = 8
 ERR_INDEX_OUT_OF_RANGE = 9
 
-SCORE_AUTO, SCORE_L_CLASSIC, SCORE_L_U32, SCORE_P = 0, 2, 3, 4
+SCORE_AUTO, SCORE_L_SCALAR, SCORE_L_CLASSIC, SCORE_L_U32, SCORE_P = 0, 1, 2, 3, 4
 
 # every symbol include/turbovec_hip.h declares
 EXPORTS = [

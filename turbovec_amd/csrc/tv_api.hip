@@ -171,6 +171,11 @@ int upload_tables(tv_index *ix) {
     return TV_OK;
 }
 
+int effective_mode(const tv_index *ix);
+// Queries one LUT-scan launch serves: the scalar definition's float chain runs one query at a time.
+int lut_tile_q(const tv_index *ix, int k) { return effective_mode(ix) == TV_SCORE_L_SCALAR ? 1 : tv::lut_tile_queries(ix->geo.nch, k); }
+int lut_append_q(const tv_index *ix) { return effective_mode(ix) == TV_SCORE_L_SCALAR ? 1 : tv::lut_append_queries(ix->geo.nch); }
+
 int effective_mode(const tv_index *ix) {
     int m = ix->score_mode;
     if (m == TV_SCORE_AUTO) m = ix->geo.bits == 4 ? TV_SCORE_P : TV_SCORE_L_U32;
@@ -251,7 +256,8 @@ void fill_scan_args(const tv_index *ix, tv::ScanArgs &a) {
     a.n_blocks = uint32_t((ix->n + tv::kVecBlock - 1) / tv::kVecBlock);
     a.nch = ix->geo.nch;
     std::memcpy(a.lv, ix->levels, 16);
-    a.classic = effective_mode(ix) == TV_SCORE_L_CLASSIC;
+    a.classic = effective_mode(ix) == TV_SCORE_L_CLASSIC ? 1 : effective_mode(ix) == TV_SCORE_L_SCALAR ? 2 : 0;
+    a.n_groups = ix->geo.G;
     a.b_step = 1;
 }
 
@@ -280,7 +286,7 @@ size_t robust_need(const tv_index *ix, size_t cq, size_t k_eff) {
     const bool mode_p = effective_mode(ix) == TV_SCORE_P;
     const bool lists = k_eff <= size_t(tv::kMaxListK);
     const int kl = lists ? int(k_eff) : 1;
-    const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_tile_queries(g.nch, kl));
+    const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(lut_tile_q(ix, kl));
     const size_t n_tiles = (cq + tile_q - 1) / tile_q;
     const int grid = tv::scan_grid_blocks(ix->device, mode_p, g.nch, kl, int(tile_q));
     const size_t total_threads = size_t(grid) * tv::kScanThreads;
@@ -302,7 +308,7 @@ SampledPlan sampled_plan(const tv_index *ix, size_t cq) {
     const tv::Geometry &g = ix->geo;
     const bool mode_p = effective_mode(ix) == TV_SCORE_P;
     SampledPlan p;
-    p.tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_append_queries(g.nch));
+    p.tile_q = mode_p ? size_t(tv::kQTile) : size_t(lut_append_q(ix));
     p.n_tiles = (cq + p.tile_q - 1) / p.tile_q;
     p.cq_pad = p.n_tiles * p.tile_q;
     // large chunks of high-dimensional queries take the wide kernel: all of them in one pass per level
@@ -402,7 +408,7 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
     for (size_t q0 = 0; q0 < nq; q0 += kChunkQueries) {
         const size_t cq = std::min(kChunkQueries, nq - q0);
         const int kl = lists ? int(k_eff) : 1;
-        const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_tile_queries(g.nch, kl));
+        const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(lut_tile_q(ix, kl));
         const size_t n_tiles = (cq + tile_q - 1) / tile_q;
         const int grid = tv::scan_grid_blocks(ix->device, mode_p, g.nch, kl, int(tile_q));
         const size_t total_threads = size_t(grid) * tv::kScanThreads;
@@ -452,7 +458,7 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
             float *os = d_out_scores + (q0 + t * tile_q) * k_eff;
             int64_t *oi = d_out_idx + (q0 + t * tile_q) * k_eff;
             if (lists) {
-                const int qmod = mode_p ? tv::kQTile : tv::lut_launch_ql(g.nch, kl, a.nq_tile);
+                const int qmod = mode_p ? tv::kQTile : mode == TV_SCORE_L_SCALAR ? 1 : tv::lut_launch_ql(g.nch, kl, a.nq_tile);
                 TV_HIP(tv::launch_merge(d_part_s, d_part_i, d_part_c, int(total_threads), qmod, int(k_eff), int(k_eff),
                                         a.nq_tile, os, oi, nullptr, ix->stream));
             } else {
@@ -1087,7 +1093,7 @@ int tv_index_set_calibration(tv_index *ix, const float *shift, const float *scal
 
 int tv_index_set_score_mode(tv_index *ix, int mode) {
     if (!ix) return TV_ERR_BAD_ARGUMENT;
-    if (mode != TV_SCORE_AUTO && mode != TV_SCORE_L_CLASSIC && mode != TV_SCORE_L_U32 && mode != TV_SCORE_P)
+    if (mode != TV_SCORE_AUTO && mode != TV_SCORE_L_SCALAR && mode != TV_SCORE_L_CLASSIC && mode != TV_SCORE_L_U32 && mode != TV_SCORE_P)
         return TV_ERR_BAD_ARGUMENT;
     if (mode == TV_SCORE_P && ix->geo.bits != 4) { g_last_error = "score mode P needs 4-bit codes"; return TV_ERR_BAD_ARGUMENT; }
     std::lock_guard<std::mutex> lock(ix->mu);
@@ -1432,7 +1438,7 @@ int tv_debug_scan(tv_index *ix, const float *queries, size_t nq, int32_t *acc_ou
     const tv::Geometry &g = ix->geo;
     const int mode = effective_mode(ix);
     const bool mode_p = mode == TV_SCORE_P;
-    const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(tv::lut_tile_queries(g.nch, 1));
+    const size_t tile_q = mode_p ? size_t(tv::kQTile) : size_t(lut_tile_q(ix, 1));
     for (size_t q0 = 0; q0 < nq; q0 += tile_q) {
         const size_t cq = std::min<size_t>(tile_q, nq - q0);
         size_t need = prepare_bytes(ix, cq) + round_up(cq * g.dim * 4, 256) + 2 * round_up(cq * n * 4, 256) + 65536;

@@ -61,7 +61,8 @@ struct ScanArgs {
     int *part_cnt;             // [total_threads]
     int32_t *acc_out;          // dump mode: [nq_tile][n] (may be null)
     float *score_out;          // dump mode: [nq_tile][n]
-    int classic;               // mode L: 1 = fma flush per 256 groups, 0 = u32 epilogue
+    int classic;               // mode L: 0 = u32 epilogue, 1 = fma flush per 256 groups, 2 = the scalar definition's chain of adds
+    int n_groups;              // byte groups of a row that carry codes (the rest of the last chunks is padding)
     uint32_t b_step;           // 1, or a sampling stride: only blocks j*b_step are scanned
     int share_tau;             // lists mode: waves share and raise gtau while scanning
     uint64_t *cand;            // append mode: [nq_tile][seg_stride][kSegCap] sort keys, one segment per workgroup

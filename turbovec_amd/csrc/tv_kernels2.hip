@@ -206,6 +206,12 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
         for (int qq = 0; qq < QL; ++qq) acc[qq] = 0;
         v4i macc = {0, 0, 0, 0}, macc2 = {0, 0, 0, 0};   // two chains, so that dependent MFMAs do not queue
         word_t wh[16], wl[16];
+        // The scalar definition (search.rs:3113-3128): score = bias, then for every byte group in
+        // order score += scale * hi entry, score += scale * lo entry, each a separate f32 multiply
+        // and add.  One query per launch; a vector's groups alternate between its two lanes in
+        // runs of 16, and the running sum is handed from one to the other after each run.
+        const bool scalar = QL == 1 && a.classic == 2;
+        float chain = qb[0];
         for (int c0 = 0; c0 < nch; c0 += U) {
             uint4 cur[U];
 #pragma unroll
@@ -242,9 +248,28 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
                             vh = *reinterpret_cast<const word_t *>(gbase + add_byte<e>(row_off, phi) + j * 32 * QL);
                             vl = *reinterpret_cast<const word_t *>(gbase + add_byte<e>(row_off, plo) + (j * 32 + 16) * QL);
                         }
-                        if (MF) { wh[j] = vh; wl[j] = vl; }
-                        else LutAcc<QL>::add(acc, vh, vl);
+                        if (MF || (QL == 1 && scalar)) { wh[j] = vh; wl[j] = vl; }
+                        if (!MF) LutAcc<QL>::add(acc, vh, vl);
                     });
+                }
+                if constexpr (QL == 1) {
+                    if (scalar) {
+                        const int g0 = c * 32;
+                        auto run16 = [&](float t, int gfirst) {
+#pragma unroll
+                            for (int jj = 0; jj < 16; ++jj) {
+                                if (gfirst + jj < a.n_groups) {
+                                    t = t + qs[0] * float(uint32_t(wh[jj]));
+                                    t = t + qs[0] * float(uint32_t(wl[jj]));
+                                }
+                            }
+                            return t;
+                        };
+                        if (h == 0) chain = run16(chain, g0);
+                        chain = __shfl(chain, vi);            // the first half's sum, to both lanes of the vector
+                        if (h == 1) chain = run16(chain, g0 + 16);
+                        chain = __shfl(chain, vi + 32);       // and the second half's, back
+                    }
                 }
                 if (MF) {
                     // 16 bytes of a lane = WPA groups x QL queries; the one-hot B sums them per query
@@ -295,7 +320,8 @@ __global__ __launch_bounds__(THREADS) void k_scan_lut(ScanArgs a) {
 #pragma unroll
         for (int qq = 0; qq < QL; ++qq) {
             // classic: fa * vec_scale; u32: ((f32(acc) * scale) + bias) * vec_scale (search.rs:1174-1177)
-            score[qq] = a.classic ? fa[qq] * vs : ((float(int(total[qq])) * qs[qq]) + qb[qq]) * vs;
+            score[qq] = a.classic == 1 ? fa[qq] * vs : ((float(int(total[qq])) * qs[qq]) + qb[qq]) * vs;
+            if (QL == 1 && a.classic == 2) score[qq] = chain * vs;
         }
         if (DUMP) {
             const uint32_t slot = slot0 + vi;
@@ -492,7 +518,7 @@ __global__ __launch_bounds__(kLutBtThreads) void k_scan_lut_bt(ScanArgs a, int n
         if (h == 0 && slot < a.n && ((mw >> vi) & 1u)) {
             const float vs = a.scales[slot];
             // classic: fa * vec_scale; u32: ((f32(acc) * scale) + bias) * vec_scale (search.rs:1174-1177)
-            const float sc = a.classic ? fa * vs : ((float(int(total)) * qs) + qb) * vs;
+            const float sc = a.classic == 1 ? fa * vs : ((float(int(total)) * qs) + qb) * vs;
             if (sc >= tau) {
                 const uint32_t pos = atomicAdd(scnt, 1u);
                 if (pos < kSegCap) a.cand[size_t(blockIdx.x) * kSegCap + pos] = sort_key(sc, slot);
@@ -566,7 +592,9 @@ int lut_launch_ql(int nch, int k, int nq_tile) {
 // lut_tile_queries(nch, k) otherwise.
 hipError_t launch_scan_lut(const ScanArgs &a, int grid, int mode, hipStream_t s) {
     const bool append = mode == kModeAppend;
-    if (append && a.nq_tile == 1) {
+    const bool scalar = a.classic == 2;     // the chain of float adds: one query per launch, nibble tables
+    if (scalar && a.nq_tile != 1) return hipErrorInvalidValue;
+    if (append && a.nq_tile == 1 && !scalar) {
         // one query: byte tables for as many chunks as fit, one LDS read per code byte there
         const int n_bt = lut_bt_chunks(a.nch, grid > lut_cus ? kLdsBudgetL / 2 : kLdsBudgetL);
         if (n_bt * 2 >= a.nch) {
@@ -588,7 +616,7 @@ hipError_t launch_scan_lut(const ScanArgs &a, int grid, int mode, hipStream_t s)
     const bool dump = mode != kModeLists;   // no list storage in LDS
     const int kk = a.k;                     // the tile width is chosen for the list pass of the same search
     const int threads = append ? kLutAppendThreads : kLutListThreads;
-    int ql = append ? lut_append_queries(a.nch) : lut_tile_queries(a.nch, kk);
+    int ql = scalar ? 1 : append ? lut_append_queries(a.nch) : lut_tile_queries(a.nch, kk);
     while (ql > 1 && ql / 2 >= a.nq_tile) ql >>= 1;
     const bool in_lds = lut_lds_bytes(a.nch, kk, ql, dump, threads) <= kLdsBudgetL;
     const size_t lds = in_lds ? lut_lds_bytes(a.nch, kk, ql, dump, threads)
