@@ -40,7 +40,10 @@ def masks_for(T, n, seed):
                                       (1736, 2_501, 129), (2952, 1_203, 131),
                                       # rows beyond one wave's registers (over 48 chunks): split over wave pairs
                                       (4096, 1_501, 131), (3584, 1_203, 260), (4104, 1_001, 129), (5000, 1_003, 150),
-                                      (6144, 1_001, 140), (3200, 1_501, 1029)])
+                                      (6144, 1_001, 140), (3200, 1_501, 1029),
+                                      # more than 1024 queries at 1536 dimensions: one chunk of up to 1632 on the
+                                      # ring of five slices, up to 2048 on the ring of nine; 2100 = 2048 + 52
+                                      (1536, 2_001, 1500), (1536, 2_001, 1700), (1536, 1_501, 2100)])
 def test_wide_scan_matches_oracle(T, oracle, dim, n, nq):
     oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=dim + n))
     q = unit_gaussian(nq, dim, seed=77)
@@ -48,7 +51,7 @@ def test_wide_scan_matches_oracle(T, oracle, dim, n, nq):
     for words in masks_for(T, n, 8):
         for k in (1, 10, 100):
             s, i = ix.search(q, k, mask_words=words)
-            assert ix.queries_per_launch() == nq or nq == 1029
+            assert ix.queries_per_launch() == min(nq, 2048 if dim == 1536 else 1024)
             os_, oi = oidx.search(q, k, mask_words=words)
             assert np.array_equal(i, oi), k
             assert bits_equal(s, os_), k

@@ -366,7 +366,20 @@ SamplingSteps sampling_steps(size_t n_blocks, size_t k_floor, size_t round_block
     return steps;
 }
 
-// Queries of one call are processed in chunks of kChunkQueries; the chunks of a group are enqueued
+// The all-queries-per-pass kernel holds 16 bytes of LDS per query beside its slice ring: a call with
+// more than kChunkQueries queries left takes them up to kWideChunkQueries at a time there -- a block
+// is then loaded and decoded once per 64 query tiles instead of once per 32.
+constexpr size_t kWideChunkQueries = 2 * kChunkQueries;      // (where the instance for the row length fits that many)
+bool wide_serves(const tv_index *ix) {
+    return effective_mode(ix) == TV_SCORE_P && !ix->no_batched && !ix->no_wide && tv::wide_min_queries(ix->geo.nch) > 0;
+}
+size_t chunk_len(const tv_index *ix, size_t remaining) {
+    if (remaining > kChunkQueries && wide_serves(ix))
+        return std::min(remaining, std::min<size_t>(kWideChunkQueries, size_t(tv::wide_max_queries(ix->geo.nch))));
+    return std::min(remaining, kChunkQueries);
+}
+
+// Queries of one call are processed in chunks (chunk_len); the chunks of a group are enqueued
 // back to back and the host reads their overflow flags once, after the group's last chunk.
 constexpr size_t kGroupQueries = 8 * kChunkQueries;
 constexpr size_t kLevelFlagWords = (kGroupQueries / kChunkQueries) * SamplingSteps::kMax;   // per chunk, one word per level
@@ -376,7 +389,7 @@ constexpr size_t kLevelFlagWords = (kGroupQueries / kChunkQueries) * SamplingSte
 // packed (one chunk's worth at a time); the per-level "candidates did not fit" flags of the pass in
 // flight.
 size_t group_header_bytes(const tv_index *ix, size_t gq) {
-    const size_t cq = std::min(gq, kChunkQueries);
+    const size_t cq = std::min(gq, kWideChunkQueries);
     return 2 * round_up(gq * 4, 256) + round_up(cq * 4, 256) + round_up(cq * size_t(ix->geo.dim) * 4, 256) +
            round_up(kLevelFlagWords * 4, 256);
 }
@@ -387,10 +400,18 @@ size_t group_header_bytes(const tv_index *ix, size_t gq) {
 // more candidate segments per query; it is then cut into pieces that fit).
 constexpr size_t kRepeatPieces[] = {1024, 512, 256, 128, 96, 64, 32};
 size_t sampled_need_worst(const tv_index *ix, size_t nq) {
-    const size_t gq = std::min(nq, kGroupQueries), cq = std::min(nq, kChunkQueries);
-    size_t need = sampled_plan(ix, cq).need;
-    if (nq > kChunkQueries && nq % kChunkQueries != 0) need = std::max(need, sampled_plan(ix, nq % kChunkQueries).need);
-    need = std::max(need, sampled_plan(ix, std::min<size_t>(cq, tv::kQTile)).need);
+    const size_t gq = std::min(nq, kGroupQueries);
+    size_t need = 0;
+    auto chunks_of_group = [&](size_t group_queries) {
+        for (size_t c0 = 0; c0 < group_queries;) {
+            const size_t cq = chunk_len(ix, group_queries - c0);
+            need = std::max(need, sampled_plan(ix, cq).need);
+            c0 += cq;
+        }
+    };
+    chunks_of_group(gq);                                                              // a full group, or the only one
+    if (nq > kGroupQueries && nq % kGroupQueries != 0) chunks_of_group(nq % kGroupQueries);   // and the last, shorter one
+    need = std::max(need, sampled_plan(ix, std::min<size_t>(nq, tv::kQTile)).need);
     return need + group_header_bytes(ix, gq);
 }
 
@@ -562,15 +583,19 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
         // host array (device-visible): no copy kernel between the last selection and the host's read.
         uint32_t *d_over_all = ix->d_flags_host;
         head.take<uint32_t>(gq);
-        uint32_t *d_rows = head.take<uint32_t>(std::min(gq, kChunkQueries));
-        float *d_redo_q = head.take<float>(std::min(gq, kChunkQueries) * g.dim);
+        uint32_t *d_rows = head.take<uint32_t>(std::min(gq, kWideChunkQueries));
+        float *d_redo_q = head.take<float>(std::min(gq, kWideChunkQueries) * g.dim);
+        // the group's chunks: (first query, relative to the group; length)
+        size_t chunk_at[kGroupQueries / kChunkQueries + 1], n_chunks = 0;
+        for (size_t c0 = 0; c0 < gq; c0 += chunk_len(ix, gq - c0)) chunk_at[n_chunks++] = c0;
+        chunk_at[n_chunks] = gq;
         uint32_t *d_level_flags_all = head.take<uint32_t>(kLevelFlagWords);
         size_t n_timed = 0;
 
         // One pass over `pq_n` queries of the chunk at q0: the ladder from open floors, or, for the
         // packed batch of queries to repeat (rows d_rows[row0 ..]), the ladder again from the floors
         // the pass before raised for them.  Enqueues only; the caller synchronises.
-        auto pass = [&](size_t q0, size_t row0, size_t pq_n, bool repeat, bool timed_pass) -> int {
+        auto pass = [&](size_t q0, size_t row0, size_t pq_n, bool repeat, bool timed_pass, size_t chunk_no) -> int {
             const float *d_q = d_queries + q0 * g.dim;
             float *d_os = d_out_scores + q0 * k_eff;
             int64_t *d_oi = d_out_idx + q0 * k_eff;
@@ -580,7 +605,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             const int grid = plan.grid;
             const SamplingSteps steps = level_strides(ix, plan, n_blocks, k_floor, repeat);
             const bool best_first = !repeat && first_level_is_best_of_block(ix, plan, k_floor) && steps.size() > 1;
-            uint32_t *d_level_flags = d_level_flags_all + ((q0 - g0) / kChunkQueries) * SamplingSteps::kMax;
+            uint32_t *d_level_flags = d_level_flags_all + chunk_no * SamplingSteps::kMax;
             if (head.used + plan.need > ix->ws_bytes) {
                 g_last_error = "internal: workspace smaller than the pass it was sized for";
                 return TV_ERR_BAD_ARGUMENT;
@@ -608,7 +633,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             const int bgrid = tv::batched_grid_blocks(ix->device, g.nch);
             const bool batched = nt_batched > 0 && !wide;
             const size_t tiles_per_launch = wide ? n_tiles : batched ? size_t(nt_batched) : 1;
-            if (!repeat) ix->last_queries_per_launch = int(std::min(pq_n, tile_q * tiles_per_launch));
+            if (!repeat && q0 == 0) ix->last_queries_per_launch = int(std::min(pq_n, tile_q * tiles_per_launch));   // the call's first chunk
             for (size_t lv = 0; lv < steps.size(); ++lv) {
                 const bool last = lv + 1 == steps.size();
                 // Sampling levels only yield floors, never slots, so the shifted origin of a repeated
@@ -681,8 +706,8 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
         };
 
         // first passes of every chunk of the group, back to back; one read of the flags at the end
-        for (size_t c0 = 0; c0 < gq; c0 += kChunkQueries) {
-            rc = pass(g0 + c0, 0, std::min(kChunkQueries, gq - c0), false, timing && c0 == 0);
+        for (size_t c = 0; c < n_chunks; ++c) {
+            rc = pass(g0 + chunk_at[c], 0, chunk_at[c + 1] - chunk_at[c], false, timing && c == 0, c);
             if (rc != TV_OK) return rc;
         }
         if (track_levels)
@@ -690,11 +715,11 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
         TV_HIP(hipStreamSynchronize(ix->stream));
         if (track_levels) {
             // flags of levels the passes above did not use hold whatever the workspace held: count only the used ones
-            for (size_t c0 = 0; c0 < gq; c0 += kChunkQueries) {
-                const SampledPlan plan = sampled_plan(ix, std::min(kChunkQueries, gq - c0));
+            for (size_t c = 0; c < n_chunks; ++c) {
+                const SampledPlan plan = sampled_plan(ix, chunk_at[c + 1] - chunk_at[c]);
                 const size_t n_levels = level_strides(ix, plan, n_blocks, k_floor, false).size();
                 for (size_t lv = 1; lv + 1 < n_levels; ++lv)
-                    ix->level_repeats += h_over[kGroupQueries + (c0 / kChunkQueries) * SamplingSteps::kMax + lv] != 0u;
+                    ix->level_repeats += h_over[kGroupQueries + c * SamplingSteps::kMax + lv] != 0u;
             }
         }
         for (size_t t = 0; t < n_timed; ++t) {
@@ -717,18 +742,19 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
         for (size_t i = 0; i < redo_rows.size();) {
             // rows of one chunk go together: all of them in one pass when the workspace holds that
             // pass, else in the largest pieces it holds
-            const size_t chunk = redo_rows[i] / kChunkQueries;
+            size_t chunk = 0;
+            while (chunk_at[chunk + 1] <= redo_rows[i]) ++chunk;
             size_t e = i;
-            while (e < redo_rows.size() && redo_rows[e] / kChunkQueries == chunk) ++e;
+            while (e < redo_rows.size() && redo_rows[e] < chunk_at[chunk + 1]) ++e;
             size_t piece = std::min<size_t>(e - i, tv::kQTile);
             for (size_t cand_piece : kRepeatPieces) {
                 const size_t m = std::min(cand_piece, e - i);
                 if (sampled_plan(ix, m).need <= room) { piece = m; break; }
             }
-            for (size_t r = 0; r < piece; ++r) h_over[r] = redo_rows[i + r] - uint32_t(chunk * kChunkQueries);   // pinned staging
+            for (size_t r = 0; r < piece; ++r) h_over[r] = redo_rows[i + r] - uint32_t(chunk_at[chunk]);   // pinned staging
             TV_HIP(hipMemcpyAsync(d_rows, h_over, piece * sizeof(uint32_t), hipMemcpyHostToDevice, ix->stream));
             TV_HIP(hipStreamSynchronize(ix->stream));
-            rc = pass(g0 + chunk * kChunkQueries, 0, piece, true, false);
+            rc = pass(g0 + chunk_at[chunk], 0, piece, true, false, chunk);
             if (rc != TV_OK) return rc;
             TV_HIP(hipStreamSynchronize(ix->stream));
             for (size_t r = 0; r < piece; ++r)
@@ -1392,7 +1418,7 @@ int tv_search_dev_noalloc(tv_index *ix, const float *d_queries, size_t nq, size_
     // falls back to when its candidates overflow.  Refused up front when that exceeds the array.
     size_t need = 0;
     if (k_eff != 0 && nq != 0) {
-        const size_t cq = std::min(nq, kChunkQueries);
+        const size_t cq = std::min(nq, kChunkQueries);    // the exact path works in chunks of this size throughout
         need = robust_need(ix, cq, k_eff);
         if (k_eff <= size_t(tv::kMaxSampledK) && !ix->force_robust) need = std::max(need, sampled_need_worst(ix, nq));
     }
@@ -1677,7 +1703,7 @@ int tv_debug_sampling_plan(const tv_index *cix, size_t nq, size_t k, uint32_t *s
     const size_t k_eff = std::min(k, ix->n);
     if (k_eff == 0 || nq == 0 || k_eff > size_t(tv::kMaxSampledK) || ix->force_robust) return TV_OK;   // no ladder
     const size_t n_blocks = (ix->n + tv::kVecBlock - 1) / tv::kVecBlock;
-    const SampledPlan plan = sampled_plan(ix, std::min(nq, kChunkQueries));
+    const SampledPlan plan = sampled_plan(ix, chunk_len(ix, nq));
     const SamplingSteps steps = level_strides(ix, plan, n_blocks, std::max<size_t>(k_eff, 16), false);
     *count = steps.size();
     for (size_t i = 0; i < steps.size() && i < cap; ++i) {

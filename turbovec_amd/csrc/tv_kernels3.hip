@@ -22,6 +22,8 @@
 // differs, and the candidate segments make the result independent of it.  The
 // float epilogue is skipped for a tile whose accumulators all stay below an
 // integer bound that no passing score can stay below (WideQuery).
+#include <algorithm>
+
 #include "tv_device.h"
 #include "tv_internal.h"
 
@@ -29,7 +31,9 @@ namespace tv {
 
 constexpr int kWideThreads = 512;    // the widest form (and the matrix-unit probe): 8 waves, 2 per SIMD
 constexpr int kWideWaves = kWideThreads / 64;
-constexpr int kWideRing = 5;         // LDS slots of one slice each; kWideRing - 1 slices are requested ahead
+// LDS slots of one slice each: five when slices are handed over one by one (four requested ahead) or
+// two at a time, 2 HO + 1 when more are handed over together.
+constexpr int wide_ring(int ho) { return ho <= 2 ? 5 : 2 * ho + 1; }
 
 // 16 bytes per lane from global memory (uniform base + 16 * lane) straight into LDS at
 // lds_addr + 16 * lane (lds_addr uniform over the wave).  Counted by the vector-memory counter
@@ -83,13 +87,16 @@ __device__ __forceinline__ void mfma_settle(v16i &acc) { asm volatile("s_nop 15\
 // both sides priced in (relative 1e-5, against a few 2^-24, plus 2 for the integer conversions),
 // so comparing the largest accumulator of a lane with it never loses a candidate and lets the
 // common tile -- no candidate at all -- skip the float epilogue.
+// 24 bytes per query, in two arrays: what every tile reads (the bound, with the query's scale and
+// bias beside it for the rare float score), and what only an append touches.
 struct WideQuery {
     float ta, tb;           // ta = -inf: no such bound, always score (tau <= 0, open floor, odd qs); +inf: padding query
-    uint32_t cnt;           // candidates this workgroup appended
-    float pad;
-    float qs, qb, tau;      // tau is NaN for the padding queries of the last tile: nothing passes
-    float pad2;
 };
+struct WideQueryTail {
+    float qs, qb, tau;      // tau is NaN for the padding queries of the last tile: nothing passes
+    uint32_t cnt;           // candidates this workgroup appended
+};
+constexpr int kWideQueryBytes = int(sizeof(WideQuery) + sizeof(WideQueryTail));
 
 // WAVES = 8 (two per SIMD, 256 VGPRs each) holds rows of up to 24 chunks; WAVES = 4 (one per SIMD)
 // gives a wave the whole 512-register file -- the compiler keeps what does not fit the VGPRs in
@@ -108,6 +115,7 @@ template <int NCH, int NB, int WAVES, int SPT, int BLK, int HO, int KS>
 __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide(ScanArgs a) {
     static_assert(NCH % SPT == 0, "a slice is a whole number of chunks");
     static_assert(KS == 1 || (KS == 2 && WAVES == 4 && BLK == 1 && HO == 1), "row halves go to the wave pairs of the four-wave form");
+    constexpr int kWideRing = wide_ring(HO);
     static_assert(HO == 1 || (SPT % HO == 0 && kWideRing >= 2 * HO + 1), "slices handed over together must fit the ring twice");
     extern __shared__ __align__(16) uint8_t smem[];
     if (launch_switched_off(a.run_if)) return;
@@ -131,7 +139,8 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     const int nq_pad = nt * kQTile;
     const int n_slices = SPT * nt;                          // per pass over the tiles; the host guarantees >= kAhead
     WideQuery *sq = reinterpret_cast<WideQuery *>(smem + kWideRing * kSlot);
-    float *s_vs = reinterpret_cast<float *>(sq + nq_pad);   // [waves][BLK][32]: row scales, NaN where not allowed
+    WideQueryTail *sqt = reinterpret_cast<WideQueryTail *>(sq + nq_pad);
+    float *s_vs = reinterpret_cast<float *>(sqt + nq_pad);  // [waves][BLK][32]: row scales, NaN where not allowed
     uint32_t *snext = reinterpret_cast<uint32_t *>(s_vs + kWideWaves * BLK * 32);
     v4i *s_xch = reinterpret_cast<v4i *>(snext + 16);       // KS = 2: [pairs][4][64 lanes] partial sums on their way
     const uint32_t lds_b = uint32_t(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) uint8_t *)smem));
@@ -146,10 +155,10 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
         const bool act = q < nq;
         const float qs = act ? a.qscale[q] : 0.0f, qb = act ? a.qbias[q] : 0.0f;
         const float tau = act ? order_unkey(a.gtau[q]) : __int_as_float(0x7fc00000);
-        sq[q].qs = qs;
-        sq[q].qb = qb;
-        sq[q].tau = tau;
-        sq[q].cnt = 0u;
+        sqt[q].qs = qs;
+        sqt[q].qb = qb;
+        sqt[q].tau = tau;
+        sqt[q].cnt = 0u;
         const float inf = __int_as_float(0x7f800000);
         // The bound's error analysis assumes normal floats throughout: outside 1e-30 .. 1e30
         // (subnormal floors round coarsely; tau / qs may overflow and still be met by a huge row
@@ -377,7 +386,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
         // (one or two in the whole wave, as a rule) are scored and, if they pass, appended.
         auto score_tile = [&](int q, int bound, auto kk) {
             constexpr int k = decltype(kk)::value;
-            const float4 qp = *reinterpret_cast<const float4 *>(&sq[q].qs);
+            const float4 qp = *reinterpret_cast<const float4 *>(&sqt[q].qs);
             const float qs = qp.x, qb = qp.y, tau = qp.z;
             const float *vs = s_vs + (wave * BLK + k) * 32 + 4 * h;
 #pragma unroll
@@ -386,7 +395,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
                     const int i = 8 * (r >> 2) + (r & 3);
                     const float s = fmaf(float(acc[k][r]), qs, qb) * vs[i];
                     if (s >= tau) {
-                        const uint32_t pos = atomicAdd(&sq[q].cnt, 1u);
+                        const uint32_t pos = atomicAdd(&sqt[q].cnt, 1u);
                         if (pos < kSegCap)
                             a.cand[(size_t(q) * a.seg_stride + blockIdx.x) * kSegCap + pos] =
                                 sort_key(s, blk[k] * 32u + uint32_t(i + 4 * h));
@@ -402,7 +411,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
         // reach.  One launch over a round of blocks; the hot loop never comes here.
         auto best_tile = [&](int q, auto kk) {
             constexpr int k = decltype(kk)::value;
-            const float4 qp = *reinterpret_cast<const float4 *>(&sq[q].qs);
+            const float2 qp = *reinterpret_cast<const float2 *>(&sqt[q].qs);
             const float qs = qp.x, qb = qp.y;
             const float *vs = s_vs + (wave * BLK + k) * 32 + 4 * h;
             float bs = 0.0f;
@@ -417,7 +426,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
             const int oi = __shfl_xor(bi, 32);
             if (oi >= 0 && (bi < 0 || os_ > bs || (os_ == bs && oi < bi))) { bs = os_; bi = oi; }
             if (h == 0 && bi >= 0 && q < nq) {
-                const uint32_t pos = atomicAdd(&sq[q].cnt, 1u);
+                const uint32_t pos = atomicAdd(&sqt[q].cnt, 1u);
                 if (pos < kSegCap)
                     a.cand[(size_t(q) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(bs, blk[k] * 32u + uint32_t(bi));
             }
@@ -488,7 +497,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // requests still in flight write this workgroup's LDS
     __syncthreads();
-    for (int q = tid; q < nq; q += kWideThreads) a.cand_cnt[size_t(q) * a.seg_stride + blockIdx.x] = sq[q].cnt;
+    for (int q = tid; q < nq; q += kWideThreads) a.cand_cnt[size_t(q) * a.seg_stride + blockIdx.x] = sqt[q].cnt;
 }
 
 // Matrix-unit probe: the wide kernel's MFMA loop alone -- A operands resident in registers,
@@ -577,10 +586,26 @@ int wide_blocks_per_workgroup(int nch) {
     }
 }
 
-static size_t wide_lds_bytes(int slot_bytes, int nq, int blk, int ks) {
+static size_t wide_lds_bytes(int ring, int slot_bytes, int nq, int blk, int ks) {
     const size_t nq_pad = size_t((nq + kQTile - 1) / kQTile) * kQTile;
-    return size_t(kWideRing) * slot_bytes + nq_pad * sizeof(WideQuery) + size_t(kWideWaves) * blk * 32 * 4 + 64 +
+    return size_t(ring) * slot_bytes + nq_pad * kWideQueryBytes + size_t(kWideWaves) * blk * 32 * 4 + 64 +
            (ks == 2 ? 2 * 4096 : 0);
+}
+
+// Most queries (whole tiles) a launch with this ring fits into the 160 KiB of LDS.
+static int wide_max_queries_of(int ring, int slot_bytes, int blk, int ks) {
+    const size_t fixed = wide_lds_bytes(ring, slot_bytes, 0, blk, ks);
+    if (fixed >= 160 * 1024) return 0;
+    return int((160 * 1024 - fixed) / kWideQueryBytes / kQTile * kQTile);
+}
+
+// Most queries one launch of the instance(s) for this row length serves (0: no instance); at least
+// 1024 wherever there is one.
+int wide_max_queries(int nch) {
+    switch (nch) {
+        case 24: return std::min(2048, wide_max_queries_of(wide_ring(4), 12 * 1024, 1, 1));
+        default: return wide_blocks_per_workgroup(nch) > 0 ? 1024 : 0;
+    }
 }
 
 int wide_grid_blocks(int device) {
@@ -593,7 +618,7 @@ int wide_grid_blocks(int device) {
 
 template <int NCH, int NB, int WAVES = 8, int SPT = 2, int BLK = 1, int HO = 1, int KS = 1>
 static hipError_t launch_wide_n(const ScanArgs &a, int grid, hipStream_t s) {
-    const size_t lds = wide_lds_bytes(KS * 2 * (NCH / SPT) * 1024, a.nq_tile, BLK, KS);
+    const size_t lds = wide_lds_bytes(wide_ring(HO), KS * 2 * (NCH / SPT) * 1024, a.nq_tile, BLK, KS);
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK, HO, KS>),
@@ -620,9 +645,14 @@ hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s) {
         case 14: return launch_wide_n<14, 2, 8, 2, 1, 2>(a, grid, s);
         case 16: return launch_wide_n<16, 4, 8, 2, 1, 2>(a, grid, s);
         case 18: return launch_wide_n<18, 2, 8, 2, 1, 2>(a, grid, s);
-        case 20: return launch_wide_n<20, 4, 8, 2, 1, 2>(a, grid, s);
+        case 20: return launch_wide_n<20, 2, 8, 2, 1, 2>(a, grid, s);   // (four operand registers in flight would spill one)
         case 22: return launch_wide_n<22, 2, 8, 2, 1, 2>(a, grid, s);
-        case 24: return launch_wide_n<24, 2, 8, 2, 1, 2>(a, grid, s);
+        // 24 chunks (1536 dimensions): up to 1632 queries with the ring of five 24 KiB slices; longer
+        // chunks (to 2048 queries: a block is then decoded once per 64 tiles instead of 32) with a
+        // ring of nine 12 KiB slices handed over four at a time, which leaves the LDS for them
+        case 24:
+            if (a.nq_tile <= wide_max_queries_of(wide_ring(2), 24 * 1024, 1, 1)) return launch_wide_n<24, 2, 8, 2, 1, 2>(a, grid, s);
+            return launch_wide_n<24, 2, 8, 4, 1, 4>(a, grid, s);
         case 28: return launch_wide_n<28, 2, 4, 4, 1>(a, grid, s);
         case 32: return launch_wide_n<32, 4, 4, 4, 1>(a, grid, s);
         case 36: return launch_wide_n<36, 2, 4, 4, 1>(a, grid, s);
