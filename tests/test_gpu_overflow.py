@@ -220,3 +220,39 @@ def test_unvalidated_queries_return(T, oracle, dim, nq):
         good = np.arange(nq) != 1
         assert np.array_equal(i[good], want_i[good]) and bits_equal(s[good], want_s[good]), val
     ix.close()
+
+
+@pytest.mark.parametrize("nq", [4, 130])
+def test_clustered_insertion_order_switches_to_the_row_level_ladder(T, nq):
+    """A clustered corpus inserted cluster by cluster, queries next to stored rows: a query's few
+    thousand near neighbours fill a run of consecutive blocks, of which the floorless first level
+    (one row per block) sees two or three, so its floor is far too low and the queries overflow.
+    The answer is still exact (the repeated pass), and the index then keeps to the ladder of
+    row-level samples, on which the same searches do not overflow."""
+    torch = pytest.importorskip("torch")
+    dev = torch.device("cuda:0")
+    dim, n, per_cluster, k = 768, 120_000, 4_000, 10
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(3)
+    centres = torch.randn(n // per_cluster, dim, device=dev, generator=gen)
+    cid = torch.arange(n, device=dev) // per_cluster
+    v = centres[cid] + 0.3 * torch.randn(n, dim, device=dev, generator=gen)
+    ix = T.NativeIndex(dim, 4)
+    torch.cuda.synchronize()
+    ix.add_dev(v.data_ptr(), n)
+    q = (v[:: n // nq][:nq] + 0.05 * torch.randn(nq, dim, device=dev, generator=gen)).cpu().numpy()
+    before = ix.sampling_plan(nq, k)[0].tolist()           # the floorless level and the full scan
+    assert len(before) == 2
+    s, i = ix.search(q, k)
+    first = ix.overflow_redos()
+    assert first * 8 >= nq, "the layout did not overflow the floorless level often enough: the test tests nothing"
+    assert ix.sampling_plan(nq, k)[0].tolist() != before   # switched to row-level samples (a sparser first level)
+    for _ in range(3):
+        s2, i2 = ix.search(q, k)
+        assert np.array_equal(i2, i) and bits_equal(s2, s)
+    assert ix.overflow_redos() == first and ix.exact_redos() == 0
+    ix.set_path(1)                                         # the exact path
+    s3, i3 = ix.search(q, k)
+    ix.set_path(0)
+    assert np.array_equal(i3, i) and bits_equal(s3, s)
+    ix.close()

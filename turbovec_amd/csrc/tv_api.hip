@@ -507,8 +507,9 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
 // sized so that the full scan then appends about 2048 rows per query, and reads at least
 // 8 * k_floor blocks; a quarter of the index or more is not worth sampling.
 constexpr size_t kBestLevelMaxK = 64;
+constexpr int kRowLadderSearches = 64;   // searches that keep to the row-level ladder after the floorless level failed
 bool first_level_is_best_of_block(const tv_index *ix, const SampledPlan &plan, size_t k_floor) {
-    return effective_mode(ix) == TV_SCORE_P && k_floor <= kBestLevelMaxK &&
+    return effective_mode(ix) == TV_SCORE_P && k_floor <= kBestLevelMaxK && ix->row_ladder_left == 0 &&
            (plan.wide ? tv::wide_serves_best_of_block(ix->geo.nch) : plan.nt_batched == 0);
 }
 SamplingSteps level_strides(const tv_index *ix, const SampledPlan &plan, size_t n_blocks, size_t k_floor, bool repeat) {
@@ -568,6 +569,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
     const size_t n_blocks = (n + tv::kVecBlock - 1) / tv::kVecBlock;
     // sampling levels take the k_floor-th best as the floor: a deeper order statistic is steadier
     const size_t k_floor = std::max<size_t>(k_eff, 16);
+    if (ix->row_ladder_left > 0) --ix->row_ladder_left;
     uint32_t *h_over = ix->h_flags;   // pinned, one flag per query of a group, then the groups' level flags
     const bool track_levels = ix->track_levels != 0;
     // sized once for the whole call, repeated passes included: nothing is reallocated while work is in flight
@@ -738,6 +740,9 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             else if (h_over[q] != 0u) exact_rows.push_back(uint32_t(q));
         }
         ix->overflow_redos += redo_rows.size() + exact_rows.size();
+        if (first_level_is_best_of_block(ix, sampled_plan(ix, chunk_at[1] - chunk_at[0]), k_floor) &&
+            (redo_rows.size() + exact_rows.size()) * 8 >= gq)
+            ix->row_ladder_left = kRowLadderSearches;      // from here on, the repeated passes below included
         const size_t room = ix->ws_bytes - head.used;
         for (size_t i = 0; i < redo_rows.size();) {
             // rows of one chunk go together: all of them in one pass when the workspace holds that

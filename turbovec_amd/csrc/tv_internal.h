@@ -213,6 +213,11 @@ struct tv_index {
     int no_batched = 0;            // test hook: one query tile per scan launch even for large batches
     int no_wide = 0;               // test hook: large batches go through the tile-group kernels, not the wide one
     size_t overflow_redos = 0;     // queries redone because their candidate buffer overflowed
+    // The floorless first level (best row per block) misjudges the floor when a query's neighbours
+    // sit together in a few blocks (a clustered corpus in insertion order): after a search in which
+    // it made an eighth of the queries overflow, the next searches run the ladder of row-level
+    // samples instead, and the floorless level gets another try afterwards.
+    int row_ladder_left = 0;
     int track_levels = 0;          // test hook: read the per-level flags back with the overflow flags and count them
     size_t level_repeats = 0;      // sampling levels that ran a second time because their candidates did not fit
 };
