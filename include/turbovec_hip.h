@@ -234,7 +234,8 @@ int tv_debug_queries_per_launch(const tv_index *ix, int *queries);
  * every search take the full-range list / dense-select path instead of
  * sample-then-filter; bit 1 keeps large batches on the one-tile-per-launch scan
  * instead of the batched ones; bit 2 keeps them off the all-queries-per-pass
- * kernel only. */
+ * kernel only; bit 3 keeps u8-LUT batches on the scan that holds whole tables in
+ * LDS (at most 8 queries per pass) instead of the sixteen-query one. */
 int tv_debug_set_path(tv_index *ix, int force_full_lists);
 /* The sampling ladder a search for the k best of nq queries (its first chunk of up to 1024) runs
  * on this index as it stands, unfiltered: block strides of the successive scans, strides[0 ..

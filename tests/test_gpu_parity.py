@@ -517,6 +517,36 @@ def test_all_equal_scores(T, oracle):
     ix.close()
 
 
+# ---- u8-LUT batches, u32 epilogue: sixteen queries per pass, tables streamed through LDS ----
+# 1536 x 2-bit: 12 chunks (configuration 3's row); 200 x 2-bit: 2 chunks, the second mostly padding;
+# 1000 x 2-bit: 8 chunks, rotation blocks of 8; 64 x 3-bit: one chunk (its pair is half padding);
+# 1536 x 4-bit: 24 chunks.  Query counts leave last tiles of 16, 9 (the sixteen-query scan), 8 and 1
+# (the whole-table scans).
+@pytest.mark.parametrize("dim,bits,n,nq", [(1536, 2, 20_011, 40), (1536, 2, 9_001, 25), (200, 2, 30_000, 33),
+                                           (1000, 2, 12_000, 16), (64, 3, 40_003, 48), (1536, 4, 9_001, 17)])
+def test_lut_sixteen_query_scan_matches_oracle(T, oracle, dim, bits, n, nq):
+    O = oracle
+    oidx = OracleIndex(O, dim, bits, unit_gaussian(n, dim, seed=51))
+    q = unit_gaussian(nq, dim, seed=52)
+    ix = to_native(T, oidx, tmode(T, "L_U32"))
+    rng = np.random.default_rng(7)
+    for m in (None, rng.random(n) < 0.5, rng.random(n) < 0.003, (np.arange(n) >= 5_000) & (np.arange(n) < 7_000)):
+        words = None if m is None else T.pack_mask(m)[0]
+        for k in (1, 10, 100):
+            s, i = ix.search(q, k, mask_words=words)
+            os_, oi = oidx.search(q, k, mask_words=words, mode=omode(O, "L_U32"))
+            assert np.array_equal(i, oi), k
+            assert bits_equal(s, os_), k
+            assert ix.queries_per_launch() == min(nq, 16)
+            ix.set_path(8)                        # at most 8 queries per pass, whole tables in LDS
+            s2, i2 = ix.search(q, k, mask_words=words)
+            ix.set_path(0)
+            assert np.array_equal(i2, i) and bits_equal(s2, s)
+            assert ix.queries_per_launch() <= 8
+    assert ix.overflow_redos() == 0
+    ix.close()
+
+
 # ---- batched permute-dot scan (more than 32 queries per launch) ----
 # dims 256/512/1536: weights of several tiles resident in LDS (1536 with 97 queries: the wide
 # kernel, one pass for all); 3072 and 2560: streamed in slices;

@@ -8,7 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libturbovec_hip.so")
 
-SOURCES = ["tv_kernels.hip", "tv_kernels2.hip", "tv_kernels3.hip", "tv_encode.hip", "tv_api.hip", "host_tables.cpp", "tv_snapshot.cpp"]
+SOURCES = ["tv_kernels.hip", "tv_kernels2.hip", "tv_kernels3.hip", "tv_kernels4.hip", "tv_encode.hip", "tv_api.hip", "host_tables.cpp", "tv_snapshot.cpp"]
 
 # -ffp-contract=off: the parity contract is bit-exact float arithmetic, fused
 # only where the code says fmaf.  The packed-FP32 feature is switched off for
@@ -30,7 +30,7 @@ FLAGS = [
 # a request and its wait would be read stale, silently.  So none of them may touch scratch memory.
 # (k_scan_p4, k_scan_p4_multi, k_scan_p4_wide and the matrix-unit probe; k_scan_p4_batched and the
 # LUT scans leave every wait to the compiler.)
-NO_SCRATCH = re.compile(r"k_scan_p4I|k_scan_p4_multiI|k_scan_p4_wideI|k_probe_mfma")
+NO_SCRATCH = re.compile(r"k_scan_p4I|k_scan_p4_multiI|k_scan_p4_wideI|k_scan_lut16I|k_probe_mfma")
 # These two address their byte -> levels table by the byte's value alone: the table must sit at LDS
 # address 0, i.e. the kernel may have no static LDS allocation in front of its dynamic one.
 NO_STATIC_LDS = re.compile(r"k_scan_p4(_multi)?I")

@@ -174,7 +174,15 @@ int upload_tables(tv_index *ix) {
 int effective_mode(const tv_index *ix);
 // Queries one LUT-scan launch serves: the scalar definition's float chain runs one query at a time.
 int lut_tile_q(const tv_index *ix, int k) { return effective_mode(ix) == TV_SCORE_L_SCALAR ? 1 : tv::lut_tile_queries(ix->geo.nch, k); }
-int lut_append_q(const tv_index *ix) { return effective_mode(ix) == TV_SCORE_L_SCALAR ? 1 : tv::lut_append_queries(ix->geo.nch); }
+// Queries one append-mode LUT launch serves: sixteen with the u32 epilogue (tables streamed through
+// LDS), what fits LDS whole with the classic one, one for the scalar definition's chain.
+bool lut16_serves(const tv_index *ix) { return effective_mode(ix) == TV_SCORE_L_U32 && !ix->no_lut16; }
+int lut_append_q(const tv_index *ix) {
+    if (effective_mode(ix) == TV_SCORE_L_SCALAR) return 1;
+    return lut16_serves(ix) ? tv::kLut16Queries : tv::lut_append_queries(ix->geo.nch);
+}
+// Tiles of fewer queries than this keep the whole-table scan (its pass is as long for 8 queries as for 1).
+constexpr int kLut16MinQueries = 9;
 
 int effective_mode(const tv_index *ix) {
     int m = ix->score_mode;
@@ -185,6 +193,7 @@ int effective_mode(const tv_index *ix) {
 struct Prepared {
     float *d_qrot = nullptr;   // rotated (and calibrated) rows
     uint8_t *d_tables = nullptr;
+    uint8_t *d_tables16 = nullptr;   // mode L: the same tables entry-major for the sixteen-query scan (or null)
     float *d_qscale = nullptr, *d_qbias = nullptr;
     size_t table_bytes_per_tile = 0;
 };
@@ -194,8 +203,9 @@ struct Prepared {
 // `split`: permute-dot weights in the order k_scan_p4 reads them (the batched scans take plane order)
 // `keep_rotated`: the rotated rows are wanted in device memory too (the debug read-back); a search
 // in permute-dot mode does not need them and prepares its queries in a single launch.
+// `for_append`: u8-LUT tables are wanted entry-major too, for the sixteen-query append scan.
 int prepare_queries(tv_index *ix, Arena &ar, const float *d_q, size_t nq, Prepared &out, bool split = true,
-                    bool keep_rotated = false) {
+                    bool keep_rotated = false, bool for_append = false) {
     const tv::Geometry &g = ix->geo;
     const size_t nq_pad = round_up(nq, tv::kQTile);
     const int mode = effective_mode(ix);
@@ -236,6 +246,10 @@ int prepare_queries(tv_index *ix, Arena &ar, const float *d_q, size_t nq, Prepar
         out.d_tables = ar.take<uint8_t>(nq_pad * size_t(g.nch) * 1024);
         TV_HIP(tv::launch_build_lut(d_cal, d_bias_corr, ix->d_centroids, out.d_tables, out.d_qscale, out.d_qbias,
                                     g.dim, g.bits, g.G, g.nch, nq, nq_pad, ix->stream));
+        if (for_append && lut16_serves(ix) && nq >= size_t(kLut16MinQueries)) {
+            out.d_tables16 = ar.take<uint8_t>(tv::lut16_table_bytes(g.nch, nq));
+            TV_HIP(tv::launch_lut_interleave16(out.d_tables, out.d_tables16, g.nch, nq, ix->stream));
+        }
     }
     return TV_OK;
 }
@@ -245,6 +259,7 @@ size_t prepare_bytes(const tv_index *ix, size_t nq) {
     const size_t nq_pad = round_up(nq, tv::kQTile);
     size_t b = 2 * round_up(nq * g.dim * 4, 256) + 3 * round_up(nq_pad * 4, 256);
     b += round_up(nq_pad * size_t(g.nch) * 1024, 256) + 4096;
+    if (lut16_serves(ix)) b += round_up(tv::lut16_table_bytes(g.nch, nq), 256);
     return b;
 }
 
@@ -624,7 +639,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             Prepared pq;
             const int nt_batched = plan.nt_batched;
             int prc = prepare_queries(ix, ar, repeat ? d_redo_q : d_q, pq_n, pq,
-                                      !wide && (nt_batched == 0 || tv::batched_weights_split(g.nch)));
+                                      !wide && (nt_batched == 0 || tv::batched_weights_split(g.nch)), false, true);
             if (prc != TV_OK) return prc;
             uint64_t *d_cand = ar.take<uint64_t>(cq_pad * seg_stride * tv::kSegCap);
             uint32_t *d_cnt = ar.take<uint32_t>(cq_pad * seg_stride);
@@ -688,6 +703,9 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
                             TV_HIP(tv::launch_scan_p4_batched(a, n_seg, ix->stream));
                         } else if (mode_p) {
                             TV_HIP(tv::launch_scan_p4(a, lgrid, (best_first && lv == 0) ? tv::kModeBest : tv::kModeAppend, ix->stream));
+                        } else if (pq.d_tables16 != nullptr && a.nq_tile >= kLut16MinQueries) {
+                            a.tables = pq.d_tables16 + t * tv::lut16_table_bytes(g.nch, tile_q);
+                            TV_HIP(tv::launch_scan_lut16(a, lgrid, ix->stream));
                         } else {
                             TV_HIP(tv::launch_scan_lut(a, lgrid, tv::kModeAppend, ix->stream));
                         }
@@ -1696,6 +1714,7 @@ int tv_debug_set_path(tv_index *ix, int force_full_lists) {
     ix->force_robust = (force_full_lists & 1) != 0;
     ix->no_batched = (force_full_lists & 2) != 0;
     ix->no_wide = (force_full_lists & 4) != 0;
+    ix->no_lut16 = (force_full_lists & 8) != 0;
     return TV_OK;
 }
 

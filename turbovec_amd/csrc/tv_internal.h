@@ -112,6 +112,12 @@ int lut_tile_queries(int nch, int k);
 int lut_launch_ql(int nch, int k, int nq_tile);
 int lut_append_queries(int nch);
 int lut_append_grid(int device, int nch);
+// Sixteen queries per append-mode pass, score mode L with the u32 epilogue (tv_kernels4.hip): the
+// tables entry-major, 16 bytes per entry, two chunks (32 KiB) after another; chunks padded to even.
+constexpr int kLut16Queries = 16;
+size_t lut16_table_bytes(int nch, size_t nq);
+hipError_t launch_lut_interleave16(const uint8_t *d_src, uint8_t *d_dst, int nch, size_t nq, hipStream_t s);
+hipError_t launch_scan_lut16(const ScanArgs &a, int grid, hipStream_t s);
 hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s);
 hipError_t launch_scan_lut(const ScanArgs &a, int grid, int mode, hipStream_t s);
 // Query tiles one batched permute-dot launch serves for this geometry (0: not available).
@@ -211,6 +217,7 @@ struct tv_index {
     int last_queries_per_launch = 0;   // queries one full-scan launch of the last search served
     int force_robust = 0;          // test hook: skip sample-then-filter
     int no_batched = 0;            // test hook: one query tile per scan launch even for large batches
+    int no_lut16 = 0;              // test hook: mode L batches stay on the scan with whole tables in LDS (8 queries per pass at most)
     int no_wide = 0;               // test hook: large batches go through the tile-group kernels, not the wide one
     size_t overflow_redos = 0;     // queries redone because their candidate buffer overflowed
     // The floorless first level (best row per block) misjudges the floor when a query's neighbours
