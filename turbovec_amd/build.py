@@ -28,8 +28,8 @@ FLAGS = [
 # The scan kernels request LDS and global loads through inline assembly the compiler's wait-count
 # bookkeeping does not see, and wait for them by hand: a register spilled or reloaded between such
 # a request and its wait would be read stale, silently.  So none of them may touch scratch memory.
-# (k_scan_p4, k_scan_p4_multi, k_scan_p4_wide and the matrix-unit probe; k_scan_p4_batched and the
-# LUT scans leave every wait to the compiler.)
+# (k_scan_p4, k_scan_p4_multi, k_scan_p4_wide, k_scan_lut16 and the matrix-unit probe;
+# k_scan_p4_batched and the other LUT scans leave every wait to the compiler.)
 NO_SCRATCH = re.compile(r"k_scan_p4I|k_scan_p4_multiI|k_scan_p4_wideI|k_scan_lut16I|k_probe_mfma")
 # These two address their byte -> levels table by the byte's value alone: the table must sit at LDS
 # address 0, i.e. the kernel may have no static LDS allocation in front of its dynamic one.
