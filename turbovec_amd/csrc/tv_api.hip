@@ -316,6 +316,7 @@ size_t robust_need(const tv_index *ix, size_t cq, size_t k_eff) {
 struct SampledPlan {
     size_t tile_q, n_tiles, cq_pad, seg_stride, need;
     bool wide;
+    bool lut16;         // u8-LUT tiles of this chunk take the sixteen-query scan
     int nt_batched;     // query tiles one launch of the tile-group kernels serves (0: one tile per launch)
     int grid;
 };
@@ -329,6 +330,7 @@ SampledPlan sampled_plan(const tv_index *ix, size_t cq) {
     // large chunks of high-dimensional queries take the wide kernel: all of them in one pass per level
     const int wide_min = tv::wide_min_queries(g.nch);
     p.wide = mode_p && !ix->no_batched && !ix->no_wide && wide_min > 0 && cq >= size_t(wide_min);
+    p.lut16 = !mode_p && lut16_serves(ix) && cq >= size_t(kLut16MinQueries);
     p.nt_batched = (mode_p && cq > size_t(tv::kQTile) && !ix->no_batched) ? tv::batched_tiles(g.nch) : 0;
     p.grid = p.wide ? tv::wide_grid_blocks(ix->device)
            : mode_p ? tv::scan_grid_blocks(ix->device, mode_p, g.nch, 0, int(p.tile_q))
@@ -544,8 +546,10 @@ SamplingSteps level_strides(const tv_index *ix, const SampledPlan &plan, size_t 
         steps.step[steps.count++] = 1;
         return steps;
     }
-    return plan.wide ? sampling_steps(n_blocks, k_floor, size_t(plan.grid) * tv::wide_blocks_per_workgroup(ix->geo.nch))
-                     : sampling_steps(n_blocks, k_floor);
+    // (the sixteen-query LUT scan works in rounds too: every wave of the grid carries two blocks through the row)
+    return plan.wide    ? sampling_steps(n_blocks, k_floor, size_t(plan.grid) * tv::wide_blocks_per_workgroup(ix->geo.nch))
+           : plan.lut16 ? sampling_steps(n_blocks, k_floor, size_t(plan.grid) * tv::lut16_blocks_per_workgroup())
+                        : sampling_steps(n_blocks, k_floor);
 }
 // Block offset of a repeated pass's level of stride `step`: it samples other blocks than the pass
 // that misjudged the floor, half a stride in (an even number of blocks, so that mask words stay
@@ -670,7 +674,11 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
                     const uint32_t *run_if = attempt == 0 ? nullptr : lv_flag;
                     int n_seg = lgrid;
                     size_t launch_no = 0;
-                    for (size_t t = 0; t < n_tiles; t += tiles_per_launch, ++launch_no) {
+                    // sampling levels of the sixteen-query LUT scan: all the chunk's tiles it serves in one
+                    // launch, side by side (one tile leaves most of the chip idle for a round's time)
+                    const size_t side_by_side = (plan.lut16 && !last && pq.d_tables16 != nullptr)
+                                                    ? pq_n / tile_q + (pq_n % tile_q >= size_t(kLut16MinQueries) ? 1 : 0) : 0;
+                    for (size_t t = 0; t < n_tiles; t += (t < side_by_side ? side_by_side : tiles_per_launch), ++launch_no) {
                         tv::ScanArgs a;
                         fill_scan_args(ix, a);
                         a.mask = d_mask;
@@ -703,9 +711,13 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
                             TV_HIP(tv::launch_scan_p4_batched(a, n_seg, ix->stream));
                         } else if (mode_p) {
                             TV_HIP(tv::launch_scan_p4(a, lgrid, (best_first && lv == 0) ? tv::kModeBest : tv::kModeAppend, ix->stream));
+                        } else if (t < side_by_side) {
+                            a.tables = pq.d_tables16;
+                            a.nq_tile = int(std::min<size_t>(pq_n, side_by_side * tile_q));
+                            TV_HIP(tv::launch_scan_lut16(a, lgrid, int(side_by_side), ix->stream));
                         } else if (pq.d_tables16 != nullptr && a.nq_tile >= kLut16MinQueries) {
                             a.tables = pq.d_tables16 + t * tv::lut16_table_bytes(g.nch, tile_q);
-                            TV_HIP(tv::launch_scan_lut16(a, lgrid, ix->stream));
+                            TV_HIP(tv::launch_scan_lut16(a, lgrid, 1, ix->stream));
                         } else {
                             TV_HIP(tv::launch_scan_lut(a, lgrid, tv::kModeAppend, ix->stream));
                         }

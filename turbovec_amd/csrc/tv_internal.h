@@ -117,7 +117,8 @@ int lut_append_grid(int device, int nch);
 constexpr int kLut16Queries = 16;
 size_t lut16_table_bytes(int nch, size_t nq);
 hipError_t launch_lut_interleave16(const uint8_t *d_src, uint8_t *d_dst, int nch, size_t nq, hipStream_t s);
-hipError_t launch_scan_lut16(const ScanArgs &a, int grid, hipStream_t s);
+hipError_t launch_scan_lut16(const ScanArgs &a, int grid, int tiles, hipStream_t s);
+int lut16_blocks_per_workgroup();   // blocks one workgroup carries through a round of the row's chunks
 hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s);
 hipError_t launch_scan_lut(const ScanArgs &a, int grid, int mode, hipStream_t s);
 // Query tiles one batched permute-dot launch serves for this geometry (0: not available).

@@ -90,6 +90,19 @@ __global__ __launch_bounds__(kLut16Threads) void k_scan_lut16(ScanArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, kb = lane >> 4;
     const int nch = a.nch, npairs = (nch + 1) / 2;
+    // blockIdx.y = tile of sixteen queries: a launch may serve several tiles side by side (sampling
+    // levels, which leave most of the chip idle one tile at a time); a.nq_tile counts all their queries
+    if (blockIdx.y != 0) {
+        const size_t ty = blockIdx.y;
+        a.tables += ty * size_t(npairs) * kLut16PairBytes;
+        a.qscale += ty * kLut16Queries;
+        a.qbias += ty * kLut16Queries;
+        a.gtau += ty * kQTile;
+        a.cand += ty * kLut16Queries * a.seg_stride * kSegCap;
+        a.cand_cnt += ty * kLut16Queries * a.seg_stride;
+        a.nq_tile -= int(ty) * kLut16Queries;
+    }
+    if (a.nq_tile > kLut16Queries) a.nq_tile = kLut16Queries;
     uint32_t *scnt = reinterpret_cast<uint32_t *>(smem + 2 * kLut16PairBytes);   // candidates per query of this workgroup
     if (tid < kLut16Queries) scnt[tid] = 0u;
 
@@ -240,14 +253,20 @@ __global__ __launch_bounds__(kLut16Threads) void k_scan_lut16(ScanArgs a) {
     if (tid < a.nq_tile) a.cand_cnt[size_t(tid) * a.seg_stride + blockIdx.x] = scnt[tid];
 }
 
-// One append-mode launch over 9 to 16 queries; a.tables = the tile's interleaved tables
-// (k_lut_interleave16), a.classic must be 0.
-hipError_t launch_scan_lut16(const ScanArgs &a, int grid, hipStream_t s) {
-    if (a.classic != 0 || a.nq_tile < 1 || a.nq_tile > kLut16Queries) return hipErrorInvalidValue;
+constexpr int kLut16RoundBlocks = 2;   // per wave
+int lut16_blocks_per_workgroup() { return kLut16Threads / 64 * kLut16RoundBlocks; }
+
+// One append-mode launch over `tiles` tiles of sixteen queries (the last may hold fewer): a.nq_tile =
+// all their queries, a.tables = the first tile's interleaved tables (k_lut_interleave16), floors,
+// scales and candidate segments those of the first tile, the others' following at the strides of
+// the chunk's layout; a.classic must be 0.
+hipError_t launch_scan_lut16(const ScanArgs &a, int grid, int tiles, hipStream_t s) {
+    if (a.classic != 0 || tiles < 1 || a.nq_tile <= (tiles - 1) * kLut16Queries || a.nq_tile > tiles * kLut16Queries)
+        return hipErrorInvalidValue;
     const size_t lds = 2 * size_t(kLut16PairBytes) + 64;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_lut16<2>), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_lut16<kLut16RoundBlocks>), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(k_scan_lut16<2>, dim3(grid), dim3(kLut16Threads), lds, s, a);
+    hipLaunchKernelGGL(k_scan_lut16<kLut16RoundBlocks>, dim3(grid, tiles), dim3(kLut16Threads), lds, s, a);
     return hipGetLastError();
 }
 
