@@ -34,10 +34,11 @@ sys.path.insert(0, ROOT)
 # HBM bytes one launch of the dominant kernel moves (reads + writes), from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this same command, each scaled by the copy-probe factor (see profiles/).
 MEASURED_TRAFFIC = {
-    ("k_scan_p4_wide", 10_000_000, 1536, 4): 7.8248e9,    # 3,775,920 x 2 KiB fetched + 89,521 KiB written
-    ("k_scan_p4_multi", 10_000_000, 1536, 4): 7.7344e9,   # 3,774,660 x 2 KiB fetched + 3,784 KiB written
-    ("k_scan_p4", 10_000_000, 1536, 4): 7.7206e9,         # 3,769,810 x 2 KiB fetched + 58 KiB written
+    ("k_scan_p4_wide", 10_000_000, 1536, 4): 7.8244e9,    # 3,775,920 x 2 KiB fetched + 89,154 KiB written
+    ("k_scan_p4_multi", 10_000_000, 1536, 4): 7.7327e9,   # 3,774,380 x 2 KiB fetched + 2,678 KiB written
+    ("k_scan_p4", 10_000_000, 1536, 4): 7.7209e9,         # 3,769,820 x 2 KiB fetched + 344 KiB written
     ("k_scan_lut_bt", 10_000_000, 1536, 2): 3.8802e9,     # 1,894,650 x 2 KiB fetched
+    ("k_scan_lut16", 10_000_000, 1536, 2): 3.8830e9,      # 1,895,400 x 2 KiB fetched + 1,189 KiB written
     ("k_scan_lut", 10_000_000, 1536, 2): 3.8809e9,        # 1,894,970 x 2 KiB fetched
 }
 
@@ -154,7 +155,8 @@ def config3_extra(T, torch, build_index, run, args):
     for nq, steps in ((1024, max(3, args.steps // 2)), (1, max(args.steps, 15))):
         dt, scan_ms, launches, q_full = run(nq, steps, 1, ix=ix, k=k, dim=dim)
         launch_s = scan_ms * 1e-3 / max(launches, 1)
-        kern = "k_scan_lut_bt" if q_full == 1 else "k_scan_lut"     # byte tables serve single queries
+        # byte tables serve single queries; sixteen queries per pass stream their tables through LDS
+        kern = "k_scan_lut_bt" if q_full == 1 else "k_scan_lut16" if q_full > 8 else "k_scan_lut"
         res[f"batch{nq}"] = {"queries_per_s": nq * steps / dt, "ms_per_step": dt / steps * 1e3,
                              "queries_per_launch": q_full, "scan_launch_ms": launch_s * 1e3,
                              "roofline": {"bound": "hbm", "achieved": alg / launch_s / 1e9, "peak": 8000.0,
@@ -383,7 +385,7 @@ def main():
     if mode_p:
         kernel = "k_scan_p4_wide" if q_full >= 256 else "k_scan_p4_multi" if q_full > 32 else "k_scan_p4"
     else:
-        kernel = "k_scan_lut_bt" if q_full == 1 else "k_scan_lut"
+        kernel = "k_scan_lut_bt" if q_full == 1 else "k_scan_lut16" if q_full > 8 else "k_scan_lut"
     traffic = MEASURED_TRAFFIC.get((kernel, n, dim, bits))
     int8_ops = 2.0 * q_per_launch * n * dim        # multiply-adds x2 of one launch, permute-dot mode
 
