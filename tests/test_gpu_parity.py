@@ -523,7 +523,8 @@ def test_all_equal_scores(T, oracle):
 # 1536 x 4-bit: 24 chunks.  Query counts leave last tiles of 16, 9 (the sixteen-query scan), 8 and 1
 # (the whole-table scans).
 @pytest.mark.parametrize("dim,bits,n,nq", [(1536, 2, 20_011, 40), (1536, 2, 9_001, 25), (200, 2, 30_000, 33),
-                                           (1000, 2, 12_000, 16), (64, 3, 40_003, 48), (1536, 4, 9_001, 17)])
+                                           (1000, 2, 12_000, 16), (64, 3, 40_003, 48), (1536, 4, 9_001, 17),
+                                           (1120, 2, 17_000, 9)])     # 9 chunks: the last pair is half padding
 def test_lut_sixteen_query_scan_matches_oracle(T, oracle, dim, bits, n, nq):
     O = oracle
     oidx = OracleIndex(O, dim, bits, unit_gaussian(n, dim, seed=51))
@@ -543,6 +544,30 @@ def test_lut_sixteen_query_scan_matches_oracle(T, oracle, dim, bits, n, nq):
             ix.set_path(0)
             assert np.array_equal(i2, i) and bits_equal(s2, s)
             assert ix.queries_per_launch() <= 8
+    assert ix.overflow_redos() == 0
+    ix.close()
+
+
+# ---- one u8-LUT query: byte-table scan, first sampling level without floors (best row per block) ----
+@pytest.mark.parametrize("dim,bits,n,mode", [(1536, 2, 20_011, "L_U32"), (128, 2, 60_003, "L_U32"), (64, 3, 40_003, "L_U32"),
+                                             (256, 4, 30_000, "L_CLASSIC"), (1536, 4, 9_001, "L_U32")])
+def test_lut_single_query_matches_oracle(T, oracle, dim, bits, n, mode):
+    O = oracle
+    oidx = OracleIndex(O, dim, bits, unit_gaussian(n, dim, seed=61))
+    ix = to_native(T, oidx, tmode(T, mode))
+    rng = np.random.default_rng(9)
+    for qi, m in enumerate((None, rng.random(n) < 0.5, rng.random(n) < 0.003, (np.arange(n) >= 5_000) & (np.arange(n) < 7_000))):
+        q = unit_gaussian(1, dim, seed=70 + qi)
+        words = None if m is None else T.pack_mask(m)[0]
+        for k in (1, 10, 100, 128, 129):
+            s, i = ix.search(q, k, mask_words=words)
+            os_, oi = oidx.search(q, k, mask_words=words, mode=omode(O, mode))
+            assert np.array_equal(i, oi), k
+            assert bits_equal(s, os_), k
+    strides, _ = ix.sampling_plan(1, 10)
+    assert len(strides) == 2                      # one level without floors, then the full scan
+    strides, _ = ix.sampling_plan(1, 129)         # beyond the floorless level's k: the row-level ladder
+    assert len(strides) >= 2
     assert ix.overflow_redos() == 0
     ix.close()
 

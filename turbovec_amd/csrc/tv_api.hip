@@ -317,6 +317,7 @@ struct SampledPlan {
     size_t tile_q, n_tiles, cq_pad, seg_stride, need;
     bool wide;
     bool lut16;         // u8-LUT tiles of this chunk take the sixteen-query scan
+    bool lut_single;    // one u8-LUT query, served by the byte-table scan
     int nt_batched;     // query tiles one launch of the tile-group kernels serves (0: one tile per launch)
     int grid;
 };
@@ -335,6 +336,7 @@ SampledPlan sampled_plan(const tv_index *ix, size_t cq) {
     p.grid = p.wide ? tv::wide_grid_blocks(ix->device)
            : mode_p ? tv::scan_grid_blocks(ix->device, mode_p, g.nch, 0, int(p.tile_q))
                     : tv::lut_append_grid(ix->device, g.nch);
+    p.lut_single = !mode_p && cq == 1 && effective_mode(ix) != TV_SCORE_L_SCALAR && tv::lut_single_uses_byte_tables(g.nch, p.grid);
     p.seg_stride = size_t(p.grid);
     p.need = prepare_bytes(ix, cq) + round_up(p.n_tiles * tv::kQTile * 4, 256) +
              round_up(p.cq_pad * p.seg_stride * tv::kSegCap * 8, 256) + round_up(p.cq_pad * p.seg_stride * 4, 256) +
@@ -354,6 +356,7 @@ struct SamplingSteps {
     static constexpr int kMax = 32;   // levels grow at least fourfold: 2^31 slots need 16 at most
     uint32_t step[kMax];
     size_t count = 0;
+    bool best_first = false;   // the first level runs without floors and hands over the best row of every block it reads
     size_t size() const { return count; }
     uint32_t operator[](size_t i) const { return step[i]; }
 };
@@ -524,10 +527,13 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
 // sized so that the full scan then appends about 2048 rows per query, and reads at least
 // 8 * k_floor blocks; a quarter of the index or more is not worth sampling.
 constexpr size_t kBestLevelMaxK = 64;
+constexpr size_t kBestLevelMaxKLut = 128;   // (the single-query byte-table scan: configuration 3 asks for k = 100)
 constexpr int kRowLadderSearches = 64;   // searches that keep to the row-level ladder after the floorless level failed
 bool first_level_is_best_of_block(const tv_index *ix, const SampledPlan &plan, size_t k_floor) {
-    return effective_mode(ix) == TV_SCORE_P && k_floor <= kBestLevelMaxK && ix->row_ladder_left == 0 &&
-           (plan.wide ? tv::wide_serves_best_of_block(ix->geo.nch) : plan.nt_batched == 0);
+    if (ix->row_ladder_left != 0) return false;
+    if (effective_mode(ix) != TV_SCORE_P) return plan.lut_single && k_floor <= kBestLevelMaxKLut;   // u8 LUT: the single-query byte-table scan has the mode
+    if (k_floor > kBestLevelMaxK) return false;
+    return plan.wide ? tv::wide_serves_best_of_block(ix->geo.nch) : plan.nt_batched == 0;
 }
 SamplingSteps level_strides(const tv_index *ix, const SampledPlan &plan, size_t n_blocks, size_t k_floor, bool repeat) {
     if (!repeat && first_level_is_best_of_block(ix, plan, k_floor)) {
@@ -542,9 +548,14 @@ SamplingSteps level_strides(const tv_index *ix, const SampledPlan &plan, size_t 
             if (sample > round) sample -= sample % round;
             step = sample >= round ? (n_blocks + sample - 1) / sample : n_blocks / sample;
         }
-        if (sample * 4 <= n_blocks && step > 1) steps.step[steps.count++] = uint32_t(step);
-        steps.step[steps.count++] = 1;
-        return steps;
+        if (sample * 4 <= n_blocks && step > 1) {
+            steps.step[steps.count++] = uint32_t(step);
+            steps.step[steps.count++] = 1;
+            steps.best_first = true;
+            return steps;
+        }
+        // (an index too small for that level -- it would read a quarter of it or more -- takes the
+        // row-level ladder below: a full scan from open floors alone would append every row)
     }
     // (the sixteen-query LUT scan works in rounds too: every wave of the grid carries two blocks through the row)
     return plan.wide    ? sampling_steps(n_blocks, k_floor, size_t(plan.grid) * tv::wide_blocks_per_workgroup(ix->geo.nch))
@@ -625,7 +636,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             const bool wide = plan.wide;
             const int grid = plan.grid;
             const SamplingSteps steps = level_strides(ix, plan, n_blocks, k_floor, repeat);
-            const bool best_first = !repeat && first_level_is_best_of_block(ix, plan, k_floor) && steps.size() > 1;
+            const bool best_first = steps.best_first;
             uint32_t *d_level_flags = d_level_flags_all + chunk_no * SamplingSteps::kMax;
             if (head.used + plan.need > ix->ws_bytes) {
                 g_last_error = "internal: workspace smaller than the pass it was sized for";
@@ -770,7 +781,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             else if (h_over[q] != 0u) exact_rows.push_back(uint32_t(q));
         }
         ix->overflow_redos += redo_rows.size() + exact_rows.size();
-        if (first_level_is_best_of_block(ix, sampled_plan(ix, chunk_at[1] - chunk_at[0]), k_floor) &&
+        if (level_strides(ix, sampled_plan(ix, chunk_at[1] - chunk_at[0]), n_blocks, k_floor, false).best_first &&
             (redo_rows.size() + exact_rows.size()) * 8 >= gq)
             ix->row_ladder_left = kRowLadderSearches;      // from here on, the repeated passes below included
         const size_t room = ix->ws_bytes - head.used;

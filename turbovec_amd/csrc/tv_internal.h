@@ -112,6 +112,7 @@ int lut_tile_queries(int nch, int k);
 int lut_launch_ql(int nch, int k, int nq_tile);
 int lut_append_queries(int nch);
 int lut_append_grid(int device, int nch);
+bool lut_single_uses_byte_tables(int nch, int grid);
 // Sixteen queries per append-mode pass, score mode L with the u32 epilogue (tv_kernels4.hip): the
 // tables entry-major, 16 bytes per entry, two chunks (32 KiB) after another; chunks padded to even.
 constexpr int kLut16Queries = 16;

@@ -515,14 +515,32 @@ __global__ __launch_bounds__(kLutBtThreads) void k_scan_lut_bt(ScanArgs a, int n
         uint32_t mw = 0xffffffffu;
         if (a.mask != nullptr) mw = uint32_t(a.mask[b >> 1] >> ((b & 1) * 32));
         const uint32_t slot = slot0 + uint32_t(vi);
-        if (h == 0 && slot < a.n && ((mw >> vi) & 1u)) {
+        const bool allowed = h == 0 && slot < a.n && ((mw >> vi) & 1u);
+        float sc = 0.0f;
+        if (allowed) {
             const float vs = a.scales[slot];
             // classic: fa * vec_scale; u32: ((f32(acc) * scale) + bias) * vec_scale (search.rs:1174-1177)
-            const float sc = a.classic == 1 ? fa * vs : ((float(int(total)) * qs) + qb) * vs;
-            if (sc >= tau) {
-                const uint32_t pos = atomicAdd(scnt, 1u);
-                if (pos < kSegCap) a.cand[size_t(blockIdx.x) * kSegCap + pos] = sort_key(sc, slot);
+            sc = a.classic == 1 ? fa * vs : ((float(int(total)) * qs) + qb) * vs;
+        }
+        if (a.best_of_block) {
+            // A first sampling level without a floor: the block's best allowed row (score order, then
+            // the lower slot: the larger sort key), one candidate per block -- a real score of a real
+            // row, so the k-th best of these is a floor k scanned rows reach.
+            uint64_t key = allowed && sc == sc ? sort_key(sc, slot) : 0ull;
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) {
+                const uint32_t ohi = uint32_t(__shfl_xor(int(uint32_t(key >> 32)), d));
+                const uint32_t olo = uint32_t(__shfl_xor(int(uint32_t(key)), d));
+                const uint64_t o = (uint64_t(ohi) << 32) | olo;
+                key = o > key ? o : key;
             }
+            if (lane == 0 && key != 0ull) {
+                const uint32_t pos = atomicAdd(scnt, 1u);
+                if (pos < kSegCap) a.cand[size_t(blockIdx.x) * kSegCap + pos] = key;
+            }
+        } else if (allowed && sc >= tau) {
+            const uint32_t pos = atomicAdd(scnt, 1u);
+            if (pos < kSegCap) a.cand[size_t(blockIdx.x) * kSegCap + pos] = sort_key(sc, slot);
         }
         j = nj_live;
     }
@@ -580,6 +598,13 @@ static hipError_t allow_lds2(K kernel, size_t bytes) {
     if (bytes <= 48 * 1024) return hipSuccess;
     return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                int(bytes));
+}
+
+// Whether a single query's append-mode launch on a grid of `grid` workgroups goes to the byte-table
+// scan (which also serves a first level without floors, ScanArgs::best_of_block).
+bool lut_single_uses_byte_tables(int nch, int grid) {
+    const int n_bt = lut_bt_chunks(nch, grid > lut_cus ? kLdsBudgetL / 2 : kLdsBudgetL);
+    return n_bt * 2 >= nch;
 }
 
 int lut_launch_ql(int nch, int k, int nq_tile) {
