@@ -1380,17 +1380,20 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
         for (uint32_t u = 0; u < 4; ++u)
             if (ok[u]) keys[at[u]] = v[u];
     }
-    uint32_t sort_n = need <= 64u ? 64u : 2u;
+    // leading keys kept in order by the per-wave sorts and merges below (a power of two >= need), or 0: full sort
+    const uint32_t keep = need <= 64u ? 64u : need <= 128u ? 128u : need <= 256u ? 256u : 0u;
+    uint32_t sort_n = keep ? keep : 2u;
     while (sort_n < c_all) sort_n <<= 1;
     __syncthreads();
     for (uint32_t i = c_all + t; i < sort_n; i += kFinalThreads) keys[i] = 0ull;
     __syncthreads();
-    if (need <= 64u) {
+    if (keep != 0u) {
         // Few keys wanted: every wave sorts a chunk of its own, no barrier inside (LDS serves a
-        // wave's requests in order), and a tree of merges -- the 64 larger of two sorted 64s form
-        // a bitonic run, six strides sort it -- leaves the 64 best of all in front.
+        // wave's requests in order), and a tree of merges -- the `keep` larger of two sorted runs
+        // of `keep` form a bitonic run, log2(keep) strides sort it -- leaves the `keep` best of all
+        // in front.
         const uint32_t lane = uint32_t(t) & 63u, wv = uint32_t(t) >> 6;
-        const uint32_t len = max(64u, sort_n / (kFinalThreads / 64));
+        const uint32_t len = max(keep, sort_n / (kFinalThreads / 64));
         const uint32_t n_chunks = sort_n / len;
         auto wave_sync = []() {
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
@@ -1418,12 +1421,14 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
             __syncthreads();
             if (wv % (2 * step) == 0 && wv + step < n_chunks) {
                 const uint32_t at = wv * len, other = (wv + step) * len;
-                const uint64_t x = keys[at + lane], y = keys[other + 63u - lane];
-                if (x < y) keys[at + lane] = y;
+                for (uint32_t i = lane; i < keep; i += 64) {
+                    const uint64_t x = keys[at + i], y = keys[other + keep - 1u - i];
+                    if (x < y) keys[at + i] = y;
+                }
                 wave_sync();
-                for (uint32_t stride = 32; stride > 0; stride >>= 1) {
-                    if (lane < 32u) {
-                        const uint32_t lo = 2 * lane - (lane & (stride - 1));
+                for (uint32_t stride = keep / 2; stride > 0; stride >>= 1) {
+                    for (uint32_t i = lane; i < keep / 2; i += 64) {
+                        const uint32_t lo = 2 * i - (i & (stride - 1));
                         swap_down(at + lo, at + lo + stride);
                     }
                     wave_sync();
