@@ -522,20 +522,24 @@ def test_all_equal_scores(T, oracle):
 # 1000 x 2-bit: 8 chunks, rotation blocks of 8; 64 x 3-bit: one chunk (its pair is half padding);
 # 1536 x 4-bit: 24 chunks.  Query counts leave last tiles of 16, 9 (the sixteen-query scan), 8 and 1
 # (the whole-table scans).
-@pytest.mark.parametrize("dim,bits,n,nq", [(1536, 2, 20_011, 40), (1536, 2, 9_001, 25), (200, 2, 30_000, 33),
-                                           (1000, 2, 12_000, 16), (64, 3, 40_003, 48), (1536, 4, 9_001, 17),
-                                           (1120, 2, 17_000, 9)])     # 9 chunks: the last pair is half padding
-def test_lut_sixteen_query_scan_matches_oracle(T, oracle, dim, bits, n, nq):
+@pytest.mark.parametrize("dim,bits,n,nq,mode", [
+    (1536, 2, 20_011, 40, "L_U32"), (1536, 2, 9_001, 25, "L_U32"), (200, 2, 30_000, 33, "L_U32"),
+    (1000, 2, 12_000, 16, "L_U32"), (64, 3, 40_003, 48, "L_U32"), (1536, 4, 9_001, 17, "L_U32"),
+    (1120, 2, 17_000, 9, "L_U32"),            # 9 chunks: the last pair is half padding
+    (1536, 4, 9_001, 17, "L_CLASSIC"),        # the classic epilogue: three flush batches of 256 groups
+    (1536, 2, 20_011, 40, "L_CLASSIC"),       # 12 chunks: a flush after 8 and one at the end
+    (1120, 2, 17_000, 9, "L_CLASSIC"), (200, 2, 30_000, 33, "L_CLASSIC")])
+def test_lut_sixteen_query_scan_matches_oracle(T, oracle, dim, bits, n, nq, mode):
     O = oracle
     oidx = OracleIndex(O, dim, bits, unit_gaussian(n, dim, seed=51))
     q = unit_gaussian(nq, dim, seed=52)
-    ix = to_native(T, oidx, tmode(T, "L_U32"))
+    ix = to_native(T, oidx, tmode(T, mode))
     rng = np.random.default_rng(7)
     for m in (None, rng.random(n) < 0.5, rng.random(n) < 0.003, (np.arange(n) >= 5_000) & (np.arange(n) < 7_000)):
         words = None if m is None else T.pack_mask(m)[0]
         for k in (1, 10, 100):
             s, i = ix.search(q, k, mask_words=words)
-            os_, oi = oidx.search(q, k, mask_words=words, mode=omode(O, "L_U32"))
+            os_, oi = oidx.search(q, k, mask_words=words, mode=omode(O, mode))
             assert np.array_equal(i, oi), k
             assert bits_equal(s, os_), k
             assert ix.queries_per_launch() == min(nq, 16)

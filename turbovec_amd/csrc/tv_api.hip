@@ -174,9 +174,11 @@ int upload_tables(tv_index *ix) {
 int effective_mode(const tv_index *ix);
 // Queries one LUT-scan launch serves: the scalar definition's float chain runs one query at a time.
 int lut_tile_q(const tv_index *ix, int k) { return effective_mode(ix) == TV_SCORE_L_SCALAR ? 1 : tv::lut_tile_queries(ix->geo.nch, k); }
-// Queries one append-mode LUT launch serves: sixteen with the u32 epilogue (tables streamed through
-// LDS), what fits LDS whole with the classic one, one for the scalar definition's chain.
-bool lut16_serves(const tv_index *ix) { return effective_mode(ix) == TV_SCORE_L_U32 && !ix->no_lut16; }
+// Queries one append-mode LUT launch serves: sixteen with the u32 and the classic epilogues (tables
+// streamed through LDS), one for the scalar definition's chain.
+bool lut16_serves(const tv_index *ix) {
+    return (effective_mode(ix) == TV_SCORE_L_U32 || effective_mode(ix) == TV_SCORE_L_CLASSIC) && !ix->no_lut16;
+}
 int lut_append_q(const tv_index *ix) {
     if (effective_mode(ix) == TV_SCORE_L_SCALAR) return 1;
     return lut16_serves(ix) ? tv::kLut16Queries : tv::lut_append_queries(ix->geo.nch);
@@ -559,7 +561,7 @@ SamplingSteps level_strides(const tv_index *ix, const SampledPlan &plan, size_t 
     }
     // (the sixteen-query LUT scan works in rounds too: every wave of the grid carries two blocks through the row)
     return plan.wide    ? sampling_steps(n_blocks, k_floor, size_t(plan.grid) * tv::wide_blocks_per_workgroup(ix->geo.nch))
-           : plan.lut16 ? sampling_steps(n_blocks, k_floor, size_t(plan.grid) * tv::lut16_blocks_per_workgroup())
+           : plan.lut16 ? sampling_steps(n_blocks, k_floor, size_t(plan.grid) * tv::lut16_blocks_per_workgroup(effective_mode(ix) == TV_SCORE_L_CLASSIC))
                         : sampling_steps(n_blocks, k_floor);
 }
 // Block offset of a repeated pass's level of stride `step`: it samples other blocks than the pass

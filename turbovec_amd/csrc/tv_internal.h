@@ -113,13 +113,13 @@ int lut_launch_ql(int nch, int k, int nq_tile);
 int lut_append_queries(int nch);
 int lut_append_grid(int device, int nch);
 bool lut_single_uses_byte_tables(int nch, int grid);
-// Sixteen queries per append-mode pass, score mode L with the u32 epilogue (tv_kernels4.hip): the
+// Sixteen queries per append-mode pass, score mode L with the u32 or the classic epilogue (tv_kernels4.hip): the
 // tables entry-major, 16 bytes per entry, two chunks (32 KiB) after another; chunks padded to even.
 constexpr int kLut16Queries = 16;
 size_t lut16_table_bytes(int nch, size_t nq);
 hipError_t launch_lut_interleave16(const uint8_t *d_src, uint8_t *d_dst, int nch, size_t nq, hipStream_t s);
 hipError_t launch_scan_lut16(const ScanArgs &a, int grid, int tiles, hipStream_t s);
-int lut16_blocks_per_workgroup();   // blocks one workgroup carries through a round of the row's chunks
+int lut16_blocks_per_workgroup(bool classic);   // blocks one workgroup carries through a round of the row's chunks
 hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s);
 hipError_t launch_scan_lut(const ScanArgs &a, int grid, int mode, hipStream_t s);
 // Query tiles one batched permute-dot launch serves for this geometry (0: not available).

@@ -80,10 +80,13 @@ template <int N>
 __device__ __forceinline__ void lut_wait(v4i &r) {
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(r) : "n"(N) : "memory");
 }
-constexpr int kLutAhead = 6;
 
-// RB = blocks a wave carries through one round of the pairs.
-template <int RB>
+// RB = blocks a wave carries through one round of the pairs; kLutAhead = table reads it keeps in
+// flight.  CLASSIC: the classic epilogue (search.rs:516-582): the integer sums are flushed into a
+// float every 256 byte-groups -- four pairs of chunks -- with fma(scale, f32(sum), fa), fa starting
+// at the bias; the score is fa * vec_scale.  (Its sixteen running floats per block take the
+// registers of the second block and of two reads in flight.)
+template <int RB, bool CLASSIC, int kLutAhead>
 __global__ __launch_bounds__(kLut16Threads) void k_scan_lut16(ScanArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     if (launch_switched_off(a.run_if)) return;
@@ -169,12 +172,15 @@ __global__ __launch_bounds__(kLut16Threads) void k_scan_lut16(ScanArgs a) {
         }
         if (!__syncthreads_or(has[0] ? 1 : 0)) break;
         v4i acc[RB][2];
+        float fa[RB][2][4];
         uint4 cw[RB][2];
 #pragma unroll
         for (int i = 0; i < RB; ++i) {
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
                 acc[i][half] = v4i{0, 0, 0, 0};
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) fa[i][half][rr] = qb;
                 cw[i][half] = has[i] ? load_codes(blk[i], 0, half) : uint4{0u, 0u, 0u, 0u};
             }
         }
@@ -219,6 +225,19 @@ __global__ __launch_bounds__(kLut16Threads) void k_scan_lut16(ScanArgs a) {
                     if constexpr (n + kLutAhead < 64) issue(IntC<n + kLutAhead>{});
                 });
             }
+            if constexpr (CLASSIC) {
+                if ((p & 3) == 3 || p + 1 == npairs) {   // end of a 256-group batch (search.rs:529-531, 577-580)
+#pragma unroll
+                    for (int i = 0; i < RB; ++i) {
+#pragma unroll
+                        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                            for (int rr = 0; rr < 4; ++rr) fa[i][half][rr] = fmaf(qs, float(uint32_t(acc[i][half][rr])), fa[i][half][rr]);
+                            acc[i][half] = v4i{0, 0, 0, 0};
+                        }
+                    }
+                }
+            }
             tbuf[(buf ^ 1) * 2048 + tid] = s0;
             tbuf[(buf ^ 1) * 2048 + 1024 + tid] = s1;
             __syncthreads();
@@ -240,7 +259,7 @@ __global__ __launch_bounds__(kLut16Threads) void k_scan_lut16(ScanArgs a) {
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
                     const uint32_t slot = b * 32u + uint32_t(v0 + rr);
-                    const float s = ((float(acc[i][half][rr]) * qs) + qb) * vsr[rr];
+                    const float s = CLASSIC ? fa[i][half][rr] * vsr[rr] : ((float(acc[i][half][rr]) * qs) + qb) * vsr[rr];
                     if (s >= tau && slot < a.n && ((mw >> (v0 + rr)) & 1u)) {
                         const uint32_t pos = atomicAdd(&scnt[r], 1u);
                         if (pos < kSegCap) a.cand[(size_t(r) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(s, slot);
@@ -253,20 +272,25 @@ __global__ __launch_bounds__(kLut16Threads) void k_scan_lut16(ScanArgs a) {
     if (tid < a.nq_tile) a.cand_cnt[size_t(tid) * a.seg_stride + blockIdx.x] = scnt[tid];
 }
 
-constexpr int kLut16RoundBlocks = 2;   // per wave
-int lut16_blocks_per_workgroup() { return kLut16Threads / 64 * kLut16RoundBlocks; }
+constexpr int kLut16RoundBlocks = 2, kLut16RoundBlocksClassic = 1;   // per wave
+int lut16_blocks_per_workgroup(bool classic) { return kLut16Threads / 64 * (classic ? kLut16RoundBlocksClassic : kLut16RoundBlocks); }
 
 // One append-mode launch over `tiles` tiles of sixteen queries (the last may hold fewer): a.nq_tile =
 // all their queries, a.tables = the first tile's interleaved tables (k_lut_interleave16), floors,
 // scales and candidate segments those of the first tile, the others' following at the strides of
-// the chunk's layout; a.classic must be 0.
+// the chunk's layout; a.classic 0 (u32 epilogue) or 1 (classic).
 hipError_t launch_scan_lut16(const ScanArgs &a, int grid, int tiles, hipStream_t s) {
-    if (a.classic != 0 || tiles < 1 || a.nq_tile <= (tiles - 1) * kLut16Queries || a.nq_tile > tiles * kLut16Queries)
+    if ((a.classic != 0 && a.classic != 1) || tiles < 1 || a.nq_tile <= (tiles - 1) * kLut16Queries || a.nq_tile > tiles * kLut16Queries)
         return hipErrorInvalidValue;
     const size_t lds = 2 * size_t(kLut16PairBytes) + 64;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_lut16<kLut16RoundBlocks>), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+    auto launch = [&](auto kernel) -> hipError_t {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kernel, dim3(grid, tiles), dim3(kLut16Threads), lds, s, a);
+        return hipSuccess;
+    };
+    hipError_t e = a.classic == 1 ? launch(k_scan_lut16<kLut16RoundBlocksClassic, true, 6>) : launch(k_scan_lut16<kLut16RoundBlocks, false, 6>);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(k_scan_lut16<kLut16RoundBlocks>, dim3(grid, tiles), dim3(kLut16Threads), lds, s, a);
     return hipGetLastError();
 }
 
