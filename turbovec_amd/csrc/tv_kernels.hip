@@ -1739,7 +1739,10 @@ static hipError_t launch_multi(const ScanArgs &a, int grid, hipStream_t s) {
 }
 
 hipError_t launch_scan_p4_batched(const ScanArgs &a, int grid, hipStream_t s) {
-    switch (resident_tiles(a.nch)) {
+    // the instance for the tiles the launch really has: a third resident tile of padding queries
+    // would cost its MFMAs all the same
+    const int tiles = std::max(2, (a.nq_tile + kQTile - 1) / kQTile);
+    switch (std::min(resident_tiles(a.nch), tiles)) {
         case 4: return launch_multi<4>(a, grid, s);
         case 3: return launch_multi<3>(a, grid, s);
         case 2: return launch_multi<2>(a, grid, s);
