@@ -602,6 +602,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
     // sampling levels take the k_floor-th best as the floor: a deeper order statistic is steadier
     const size_t k_floor = std::max<size_t>(k_eff, 16);
     if (ix->row_ladder_left > 0) --ix->row_ladder_left;
+    if (ix->floorless_kept_left > 0) --ix->floorless_kept_left;
     uint32_t *h_over = ix->h_flags;   // pinned, one flag per query of a group, then the groups' level flags
     const bool track_levels = ix->track_levels != 0;
     // sized once for the whole call, repeated passes included: nothing is reallocated while work is in flight
@@ -783,9 +784,18 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             else if (h_over[q] != 0u) exact_rows.push_back(uint32_t(q));
         }
         ix->overflow_redos += redo_rows.size() + exact_rows.size();
-        if (level_strides(ix, sampled_plan(ix, chunk_at[1] - chunk_at[0]), n_blocks, k_floor, false).best_first &&
-            (redo_rows.size() + exact_rows.size()) * 8 >= gq)
-            ix->row_ladder_left = kRowLadderSearches;      // from here on, the repeated passes below included
+        if ((redo_rows.size() + exact_rows.size()) * 8 >= gq) {
+            if (level_strides(ix, sampled_plan(ix, chunk_at[1] - chunk_at[0]), n_blocks, k_floor, false).best_first) {
+                // from here on, the repeated passes below included -- unless the row-level ladder has just failed too
+                if (ix->floorless_kept_left == 0) ix->row_ladder_left = kRowLadderSearches;
+            } else if (ix->row_ladder_left > 0) {
+                // rows laid out against the row-level ladder as well: back to the floorless level, whose
+                // failure is the cheaper one (its full scan gives up within a few rounds), and no
+                // switching for a while
+                ix->row_ladder_left = 0;
+                ix->floorless_kept_left = kRowLadderSearches;
+            }
+        }
         const size_t room = ix->ws_bytes - head.used;
         for (size_t i = 0; i < redo_rows.size();) {
             // rows of one chunk go together: all of them in one pass when the workspace holds that

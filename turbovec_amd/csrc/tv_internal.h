@@ -225,8 +225,11 @@ struct tv_index {
     // The floorless first level (best row per block) misjudges the floor when a query's neighbours
     // sit together in a few blocks (a clustered corpus in insertion order): after a search in which
     // it made an eighth of the queries overflow, the next searches run the ladder of row-level
-    // samples instead, and the floorless level gets another try afterwards.
+    // samples instead, and the floorless level gets another try afterwards.  When the row-level
+    // ladder then fails the same way (rows laid out against its strides), the floorless level comes
+    // back at once and stays for as many searches: its failure costs less.
     int row_ladder_left = 0;
+    int floorless_kept_left = 0;
     int track_levels = 0;          // test hook: read the per-level flags back with the overflow flags and count them
     size_t level_repeats = 0;      // sampling levels that ran a second time because their candidates did not fit
 };
