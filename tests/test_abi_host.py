@@ -74,7 +74,7 @@ def test_rust_bindings_match_the_header():
 
 
 def test_integration_doc_lists_every_binding_entry_point():
-    """INTEGRATION.md names every non-diagnostic entry point of the header."""
+    """The integration guide at the repository root names every non-diagnostic entry point of the header."""
     header = open(os.path.join(ROOT, "include", "turbovec_hip.h")).read()
     doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     declared = set(re.findall(r"\b(tv_[a-z0-9_]+)\s*\(", header)) - {"tv_index"}
