@@ -64,9 +64,10 @@ def test_first_level_poisoned_repeats_the_second_level_only(T, oracle, bits, nq)
     ix.close()
 
 
-# 8 queries: the single-tile kernel, whose one sampling level keeps the best row of every block it reads
-@pytest.mark.parametrize("nq", [8, 140])
-def test_every_level_poisoned_goes_through_the_repeated_pass(T, oracle, nq):
+# 8 queries: the single-tile kernel, whose one sampling level keeps the best row of every block it reads;
+# 2-bit, 20 queries: the sixteen-query LUT scan (tiles of 16 and 4), first and repeated pass
+@pytest.mark.parametrize("bits,nq", [(4, 8), (4, 140), (2, 20)])
+def test_every_level_poisoned_goes_through_the_repeated_pass(T, oracle, bits, nq):
     """Every block any level of the first pass reads is poor: the full scan starts from a hopeless
     floor, every query overflows, the batch is scanned again from raised floors with the ladder
     shifted half a stride, and still equals the oracle."""
@@ -74,14 +75,14 @@ def test_every_level_poisoned_goes_through_the_repeated_pass(T, oracle, nq):
     rng = np.random.default_rng(4)
     u = rng.standard_normal(dim).astype(np.float32)
     u /= np.linalg.norm(u)
-    strides, offsets = ladder_for(T, dim, 4, n, nq, k)
+    strides, offsets = ladder_for(T, dim, bits, n, nq, k)
     assert len(strides) == (2 if nq == 8 else 3), strides
-    oidx = OracleIndex(oracle, dim, 4, rows_against(strides[:-1], n, dim, u, seed=5))
+    oidx = OracleIndex(oracle, dim, bits, rows_against(strides[:-1], n, dim, u, seed=5))
     q = queries_near(u, nq, dim, seed=6)
     ix = to_native(T, oidx)
     s, i = ix.search(q, k)
     assert ix.overflow_redos() == nq and ix.exact_redos() == 0
-    os_, oi = oracle.search_fast(oidx.rot, oidx.seq, oidx.scales, q, k, 4, dim, n)
+    os_, oi = oracle.search_fast(oidx.rot, oidx.seq, oidx.scales, q, k, bits, dim, n)
     assert np.array_equal(i, oi) and bits_equal(s, os_)
     ix.close()
 
