@@ -1,4 +1,4 @@
-// Scan, score mode L with the u32 epilogue, append mode, sixteen queries per pass.
+// Scan, score modes L with the u32 or the classic epilogue, append mode, sixteen queries per pass.
 //
 // The pass of k_scan_lut is bound by LDS reads -- two per code byte and lane, each fetching the
 // same table entry of all the launch's queries -- and the LDS serves a wave's 16-byte reads at
@@ -14,8 +14,9 @@
 // one row of one of the instruction's four k-blocks -- the four lanes r, r + 16, r + 32, r + 48
 // look up vector r (or r + 16, in a second accumulator) in the four quarters of a pair of chunks -- and
 // B[k][n] = (k % 16 == n) adds byte n of all four into column n: D[r][n] is vector r's sum for
-// query n, in the lane that then scores it.  Integers and float epilogue are those of
-// turbovec/src/search.rs:1174-1177 (the definition: :3113-3128), term for term.
+// query n, in the lane that then scores it.  Integers and float epilogues are those of
+// turbovec/src/search.rs:1174-1177 (u32) and :516-582 (classic; the definition: :3113-3128),
+// term for term.
 #include "tv_device.h"
 #include "tv_internal.h"
 
