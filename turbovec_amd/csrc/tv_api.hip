@@ -523,11 +523,12 @@ int search_robust(tv_index *ix, const float *d_queries, size_t nq, size_t k_eff,
 // all-queries-per-pass kernel works through the blocks in rounds of its grid, and its levels are
 // trimmed to whole rounds.
 //
-// A first pass served by the single-tile permute-dot kernel (up to 32 queries) runs one sampling
-// level only, without a floor: the scan hands over the best row of every block it reads
-// (kModeBest), and the k_floor-th best of those is the floor of the full scan.  The level is
-// sized so that the full scan then appends about 2048 rows per query, and reads at least
-// 8 * k_floor blocks; a quarter of the index or more is not worth sampling.
+// A first pass served by the single-tile permute-dot kernel (up to 32 queries), the all-queries
+// kernel or the single-query byte-table LUT scan runs one sampling level only, without a floor:
+// the scan hands over the best row of every block it reads (kModeBest), and the k_floor-th best
+// of those is the floor of the full scan.  The level is sized so that the full scan then appends
+// about 2048 rows per query (1024 on the all-queries kernel), and reads at least 8 * k_floor
+// blocks; a quarter of the index or more is not worth sampling.
 constexpr size_t kBestLevelMaxK = 64;
 constexpr size_t kBestLevelMaxKLut = 128;   // (the single-query byte-table scan: configuration 3 asks for k = 100)
 constexpr int kRowLadderSearches = 64;   // searches that keep to the row-level ladder after the floorless level failed
@@ -540,7 +541,12 @@ bool first_level_is_best_of_block(const tv_index *ix, const SampledPlan &plan, s
 SamplingSteps level_strides(const tv_index *ix, const SampledPlan &plan, size_t n_blocks, size_t k_floor, bool repeat) {
     if (!repeat && first_level_is_best_of_block(ix, plan, k_floor)) {
         SamplingSteps steps;
-        size_t sample = std::max<size_t>((n_blocks * k_floor + 2047) / 2048, 8 * k_floor);
+        // (the all-queries kernel pays for every candidate of the full scan -- a tile with one in it
+        // leaves the integer fast path -- and samples twice as many blocks for a floor that lets half
+        // as many through: 10M x 1536, 1024 queries: two rounds of its grid instead of one, +0.12 ms
+        // of sampling, -0.25 ms of scan)
+        const size_t per = plan.wide ? 1024 : 2048;
+        size_t sample = std::max<size_t>((n_blocks * k_floor + per - 1) / per, 8 * k_floor);
         sample = std::min<size_t>(sample, size_t(plan.grid) * (tv::kSegCap / 2));   // a workgroup's blocks fit its segment
         size_t step = sample ? n_blocks / sample : 0;
         if (plan.wide) {
