@@ -191,7 +191,9 @@ def adversarial_extra(T, torch, run, args, normal_ms, ladder):
         os_ = torch.empty(nq, k, device=dev)
         oi = torch.empty(nq, k, dtype=torch.int64, device=dev)
         ix.level_repeats(track=1)
+        t1 = time.perf_counter()
         ix.search_dev(q.data_ptr(), nq, k, os_.data_ptr(), oi.data_ptr())
+        first_ms, first_redos = (time.perf_counter() - t1) * 1e3, ix.overflow_redos()
         r0, e0, l0 = ix.overflow_redos(), ix.exact_redos(), ix.level_repeats()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -204,6 +206,9 @@ def adversarial_extra(T, torch, run, args, normal_ms, ladder):
         ms = (time.perf_counter() - t0) / steps * 1e3
         # (the library changes ladders when one fails for many queries, so the steps need not cost the same)
         return {"ms_per_step": ms, "vs_normal": ms / normal_ms, "ms_each_step": each,
+                # the index's first search on this layout (untimed above; it also pays first-use set-up):
+                # where a ladder fails for the first time and the library switches
+                "first_search_ms": round(first_ms, 3), "first_search_queries_repeated": first_redos,
                 "queries_repeated_per_step": (ix.overflow_redos() - r0) / steps,
                 "queries_on_exact_path_per_step": (ix.exact_redos() - e0) / steps,
                 "sampling_levels_repeated_per_step": (ix.level_repeats() - l0) / steps}
