@@ -108,7 +108,9 @@ __global__ __launch_bounds__(kLut16Threads) void k_scan_lut16(ScanArgs a) {
     }
     if (a.nq_tile > kLut16Queries) a.nq_tile = kLut16Queries;
     uint32_t *scnt = reinterpret_cast<uint32_t *>(smem + 2 * kLut16PairBytes);   // candidates per query of this workgroup
+    uint32_t *s_over = scnt + kLut16Queries;                                     // queries whose segment of this workgroup is full
     if (tid < kLut16Queries) scnt[tid] = 0u;
+    if (tid == kLut16Queries) *s_over = 0u;
 
     // the query whose column of the result this lane holds
     const bool qact = r < a.nq_tile;
@@ -165,6 +167,11 @@ __global__ __launch_bounds__(kLut16Threads) void k_scan_lut16(ScanArgs a) {
     for (;;) {
         uint32_t blk[RB];
         bool has[RB];
+        // Once every query's segment of this workgroup is full, every query of the launch is certain
+        // to be flagged as overflowed and scanned again from a raised floor: nothing this workgroup
+        // could still append would be kept, so it takes no further blocks (rows laid out against the
+        // sampler end the launch within a few rounds instead of scoring the whole index for nothing).
+        if (*reinterpret_cast<volatile uint32_t *>(s_over) >= uint32_t(a.nq_tile)) j = nj;
 #pragma unroll
         for (int i = 0; i < RB; ++i) {
             has[i] = j < nj;
@@ -264,6 +271,7 @@ __global__ __launch_bounds__(kLut16Threads) void k_scan_lut16(ScanArgs a) {
                     if (s >= tau && slot < a.n && ((mw >> (v0 + rr)) & 1u)) {
                         const uint32_t pos = atomicAdd(&scnt[r], 1u);
                         if (pos < kSegCap) a.cand[(size_t(r) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(s, slot);
+                        else if (pos == kSegCap) atomicAdd(s_over, 1u);      // the one append that finds the segment just full
                     }
                 }
             }
@@ -283,7 +291,7 @@ int lut16_blocks_per_workgroup(bool classic) { return kLut16Threads / 64 * (clas
 hipError_t launch_scan_lut16(const ScanArgs &a, int grid, int tiles, hipStream_t s) {
     if ((a.classic != 0 && a.classic != 1) || tiles < 1 || a.nq_tile <= (tiles - 1) * kLut16Queries || a.nq_tile > tiles * kLut16Queries)
         return hipErrorInvalidValue;
-    const size_t lds = 2 * size_t(kLut16PairBytes) + 64;
+    const size_t lds = 2 * size_t(kLut16PairBytes) + 128;
     auto launch = [&](auto kernel) -> hipError_t {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
         if (e != hipSuccess) return e;
