@@ -1198,18 +1198,38 @@ __device__ __forceinline__ void sort8_desc(uint64_t (&r)[8]) {
     ce(2, 4); ce(3, 5);
     ce(1, 2); ce(3, 4); ce(5, 6);
 }
-// The `need` (<= 32) largest of the wave's keys -- eight per lane, sorted descending, 0 = none,
+// Sixteen keys in descending order: two sorted eights, then a bitonic merge (70 exchanges).
+__device__ __forceinline__ void sort16_desc(uint64_t (&r)[16]) {
+    auto ce = [&](int i, int j) { if (r[i] < r[j]) { const uint64_t x = r[i]; r[i] = r[j]; r[j] = x; } };
+    uint64_t a[8], b[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { a[e] = r[e]; b[e] = r[8 + e]; }
+    sort8_desc(a);
+    sort8_desc(b);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { r[e] = a[e]; r[8 + e] = b[e]; }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ce(i, 15 - i);              // the eight larger in front, both halves bitonic
+#pragma unroll
+    for (int stride = 4; stride >= 1; stride >>= 1) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            if ((i & stride) == 0) ce(i, i + stride);
+    }
+}
+// The `need` (<= 32) largest of the wave's keys -- N per lane, sorted descending, 0 = none,
 // non-zero keys distinct -- in order: lane i returns the i-th largest (0 beyond what there is).
 // One largest key is found and retired per turn; nothing touches LDS.
-__device__ __forceinline__ uint64_t wave_top(uint64_t (&r)[8], uint32_t need, uint32_t lane) {
+template <int N>
+__device__ __forceinline__ uint64_t wave_top(uint64_t (&r)[N], uint32_t need, uint32_t lane) {
     uint64_t mine = 0ull;
     for (uint32_t it = 0; it < need; ++it) {
         const uint64_t m = wave_umax64(r[0]);
         if (lane == it) mine = m;
         if (r[0] == m && m != 0ull) {
 #pragma unroll
-            for (int e = 0; e < 7; ++e) r[e] = r[e + 1];
-            r[7] = 0ull;
+            for (int e = 0; e < N - 1; ++e) r[e] = r[e + 1];
+            r[N - 1] = 0ull;
         }
     }
     return mine;
@@ -1228,7 +1248,7 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
                                                uint32_t *clear_flag, const uint32_t *run_if) {
     __shared__ uint64_t keys[kFinalCap];
     __shared__ uint32_t wave_sum[kFinalThreads / 64];
-    __shared__ uint32_t any_full, long_n, any_long;
+    __shared__ uint32_t any_full, long_n, any_long, any_over8;
     __shared__ uint32_t long_seg[kFinalLong], long_pos[kFinalLong], long_cnt[kFinalLong];
     const int qn = blockIdx.x;
     const int t = threadIdx.x;
@@ -1236,13 +1256,13 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
     int *tau_slot = sampling ? tau_out + (qn / tau_stride_q) * kQTile + qn % tau_stride_q : nullptr;
     if (launch_switched_off(run_if)) return;
     if (clear_flag != nullptr && qn == 0 && t == 0) *clear_flag = 0u;
-    if (t == 0) { any_full = 0u; long_n = 0u; any_long = 0u; }
+    if (t == 0) { any_full = 0u; long_n = 0u; any_long = 0u; any_over8 = 0u; }
     __syncthreads();
     // every thread owns a contiguous run of this query's segments
     const uint32_t per = (n_seg + kFinalThreads - 1) / kFinalThreads;
     const uint32_t s0 = min(uint32_t(t) * per, n_seg), s1 = min(s0 + per, n_seg);
     const uint32_t *cnt = cand_cnt + size_t(qn) * seg_stride;
-    constexpr uint32_t kShort = 8;
+    constexpr uint32_t kShort = 16;
     // One segment per thread (the usual case): its head is requested together with its count, not
     // after it -- the segment's memory is there whatever the count says -- which takes one trip to
     // memory out of a kernel that is nothing but latency.
@@ -1260,6 +1280,7 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
             if (c > kSegCap) any_full = 1u;
             mine = min(c, uint32_t(kSegCap));
             if (mine > kShort) any_long = 1u;
+            if (mine > 8u) any_over8 = 1u;
         }
     } else {
         for (uint32_t sg = s0; sg < s1; ++sg) {
@@ -1313,8 +1334,17 @@ __global__ __launch_bounds__(kFinalThreads) void k_final(const uint64_t *__restr
         const uint32_t lane = uint32_t(t) & 63u, wv = uint32_t(t) >> 6;
 #pragma unroll
         for (uint32_t e = 0; e < kShort; ++e) if (e >= mine) head[e] = 0ull;
-        sort8_desc(head);
-        const uint64_t pick = wave_top(head, need, lane);
+        uint64_t pick;
+        if (any_over8 == 0u) {          // the usual case: eight keys per thread at most
+            uint64_t r8[8];
+#pragma unroll
+            for (uint32_t e = 0; e < 8; ++e) r8[e] = head[e];
+            sort8_desc(r8);
+            pick = wave_top(r8, need, lane);
+        } else {
+            sort16_desc(head);
+            pick = wave_top(head, need, lane);
+        }
         if (lane < 32u) keys[wv * 32u + lane] = pick;
         __syncthreads();
         if (wv == 0) {
