@@ -461,7 +461,7 @@ def test_sampled_path_matches_oracle_and_full_path(T, oracle, bits, mode):
     masks = [None, rng.random(n) < 0.5, rng.random(n) < 0.01, (np.arange(n) > 30_000) & (np.arange(n) < 32_000)]
     for m in masks:
         words = None if m is None else T.pack_mask(m)[0]
-        for k in (1, 10, 32, 33, 100, 1000, 1500):
+        for k in (1, 10, 32, 33, 100, 128, 200, 256, 257, 1000, 1500):   # (64, 128, 256 leading keys kept by the selection's merge tree; full sort beyond)
             s, i = ix.search(q, k, mask_words=words)
             os_, oi = oidx.search(q, k, mask_words=words, mode=omode(O, mode))
             assert np.array_equal(i, oi), (mode, k)
