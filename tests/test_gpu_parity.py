@@ -578,10 +578,11 @@ def test_lut_single_query_matches_oracle(T, oracle, dim, bits, n, mode):
 
 # ---- batched permute-dot scan (more than 32 queries per launch) ----
 # dims 256/512/1536: weights of several tiles resident in LDS (1536 with 97 queries: the wide
-# kernel, one pass for all); 3072 and 2560: streamed in slices;
+# kernel, one pass for all); 3072 and 2560: streamed in slices, by the instance for two, three
+# or four tiles of queries (45, 70, 131 queries);
 # 2624 (41 chunks, odd): no batched kernel applies, the single-tile scan serves the batch.
 @pytest.mark.parametrize("dim,n,nq", [(256, 40_003, 200), (1536, 20_011, 97), (1536, 9_001, 70), (512, 70_000, 129),
-                                      (3072, 12_345, 131), (2560, 9_001, 70), (2624, 5_003, 40)])
+                                      (3072, 12_345, 131), (2560, 9_001, 70), (3072, 7_001, 45), (2624, 5_003, 40)])
 def test_batched_scan_matches_oracle(T, oracle, dim, n, nq):
     O = oracle
     oidx = OracleIndex(O, dim, 4, unit_gaussian(n, dim, seed=41))

@@ -1778,13 +1778,22 @@ hipError_t launch_scan_p4_batched(const ScanArgs &a, int grid, hipStream_t s) {
         case 2: return launch_multi<2>(a, grid, s);
         default: break;
     }
-    constexpr int NT = kStreamTiles, MW = kStreamBlocksPerWave, KC = kStreamSliceChunks, OCC = kStreamOccupancy;
-    if (a.nch % KC != 0 || a.nq_tile > NT * kQTile) return hipErrorInvalidValue;
-    const size_t lds = size_t(2) * NT * KC * 2048 + NT * kQTile * sizeof(uint32_t);
-    hipError_t e = allow_lds(k_scan_p4_batched<NT, MW, KC, OCC>, lds);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((k_scan_p4_batched<NT, MW, KC, OCC>), dim3(grid), dim3(kScanThreads), lds, s, a);
-    return hipGetLastError();
+    constexpr int MW = kStreamBlocksPerWave, KC = kStreamSliceChunks, OCC = kStreamOccupancy;
+    if (a.nch % KC != 0 || a.nq_tile > kStreamTiles * kQTile) return hipErrorInvalidValue;
+    auto launch = [&](auto ntc) -> hipError_t {
+        constexpr int NT = decltype(ntc)::value;
+        const size_t lds = size_t(2) * NT * KC * 2048 + NT * kQTile * sizeof(uint32_t);
+        hipError_t e = allow_lds(k_scan_p4_batched<NT, MW, KC, OCC>, lds);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL((k_scan_p4_batched<NT, MW, KC, OCC>), dim3(grid), dim3(kScanThreads), lds, s, a);
+        return hipGetLastError();
+    };
+    static_assert(kStreamTiles == 4, "one instance per tile count up to the stream's four");
+    switch (tiles) {        // as above: no tile of padding queries
+        case 2: return launch(IntC<2>{});
+        case 3: return launch(IntC<3>{});
+        default: return launch(IntC<4>{});
+    }
 }
 
 hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, const int *part_cnt, int total_threads,
