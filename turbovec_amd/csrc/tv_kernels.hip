@@ -1723,7 +1723,10 @@ static int resident_tiles(int nch) {
     return nt > 4 ? 4 : nt;
 }
 
-constexpr int kMultiThreads = 768;   // 3 waves per SIMD: measured best of 512 / 768 / 1024
+// Waves per workgroup of the resident-weights kernel: three per SIMD (measured best of 512 / 768 /
+// 1024 threads with three and four tiles' accumulators); the two-tile instance fits 128 registers
+// and runs four per SIMD (2 to 7 % faster per launch, 256 to 2048 dimensions).
+template <int NT> constexpr int kMultiThreads = NT == 2 ? 1024 : 768;
 constexpr int kStreamTiles = 4, kStreamBlocksPerWave = 2, kStreamSliceChunks = 2, kStreamOccupancy = 2;
 
 // The resident-weights kernel reads its weights in k_scan_p4's split order.
@@ -1751,9 +1754,9 @@ int batched_grid_blocks(int device, int nch) {
 template <int NT, int U>
 static hipError_t launch_multi_u(const ScanArgs &a, int grid, hipStream_t s) {
     const size_t lds = kDecodeBytes + size_t(NT) * a.nch * 2048 + (NT * kQTile + 1) * sizeof(uint32_t);
-    hipError_t e = allow_lds(k_scan_p4_multi<NT, U, kMultiThreads>, lds);
+    hipError_t e = allow_lds(k_scan_p4_multi<NT, U, kMultiThreads<NT>>, lds);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((k_scan_p4_multi<NT, U, kMultiThreads>), dim3(grid), dim3(kMultiThreads), lds, s, a);
+    hipLaunchKernelGGL((k_scan_p4_multi<NT, U, kMultiThreads<NT>>), dim3(grid), dim3(kMultiThreads<NT>), lds, s, a);
     return hipGetLastError();
 }
 
