@@ -23,12 +23,12 @@ def masks_for(T, n, seed):
     return [None if m is None else T.pack_mask(m)[0] for m in out]
 
 
-# dims 1280 to 3072 switch to the wide kernel at 97 queries (2048 and up: its four-wave form, a
-# row's operands in 512 registers), dims up to 1024 at 129 (256 to 768: two to four blocks per wave); the query counts
+# dims 1280 to 2304 switch to the wide kernel at 97 queries (2048 and up: its four-wave form, a
+# row's operands in 512 registers), dims up to 1024 and from 2560 at 129 (256 to 768: two to four blocks per wave); the query counts
 # leave a ragged last tile, and 1029 = one full chunk of 1024 plus a 5-query chunk that the
 # single-tile kernel serves
 @pytest.mark.parametrize("dim,n,nq", [(1536, 6_007, 300), (1280, 4_001, 257), (1280, 3_001, 100), (1024, 5_003, 520), (1536, 3_001, 1029),
-                                      (2048, 3_001, 200), (2560, 2_001, 100), (3072, 2_501, 260),
+                                      (2048, 3_001, 200), (2560, 2_001, 140), (3072, 2_501, 260),
                                       (256, 20_011, 333), (384, 9_001, 130), (512, 12_345, 200), (768, 7_003, 290),
                                       (1024, 4_001, 129), (128, 30_011, 400), (640, 5_003, 140), (896, 4_001, 200),
                                       (1152, 3_001, 130), (1408, 3_003, 100), (1792, 2_001, 100), (2304, 2_003, 129),

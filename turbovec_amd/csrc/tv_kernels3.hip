@@ -556,13 +556,17 @@ hipError_t launch_probe_mfma(int device, int iters, uint32_t *sink, double *ops,
 // length.  Measured against the tile-group kernels on 4-bit indexes of 256 to 3072 dimensions:
 // the wide kernel wins as soon as the tile-group kernel would need a second pass over the codes
 // (it serves 128 queries per pass up to 1024 dimensions, 96 at 1280 and 1536), by 1.4 to 1.6
-// times at 1024 queries; from 2048 dimensions, where the tile-group kernel streams its weights
-// too, it is level at 128 queries and 1.6 to 1.7 times faster at 1024.
+// times at 1024 queries; at 1792 to 2304 dimensions, where two tiles' weights stay resident, it is
+// level at 97 to 128 queries (two tile-group passes); from 2560 dimensions the tile-group kernel
+// streams four tiles' weights and serves 128 queries in one pass, 1 to 7 % faster than the wide
+// kernel there, which takes over from 129 (1.2 to 1.4 times faster at 160 to 384 queries, 1.6 to
+// 1.7 times at 1024).
 int wide_min_queries(int nch) {
     switch (nch) {
         case 2: case 4: case 6: case 8: case 10: case 12: case 14: case 16: case 18: return 129;
         case 20: case 22: case 24: return 97;
-        case 28: case 32: case 36: case 40: case 44: case 48: return 97;
+        case 28: case 32: case 36: return 97;
+        case 40: case 44: case 48: return 129;
         case 56: case 64: case 72: case 80: case 88: case 96: return 129;
         default: return 0;
     }
