@@ -68,6 +68,7 @@ struct ScanArgs {
     uint64_t *cand;            // append mode: [nq_tile][seg_stride][kSegCap] sort keys, one segment per workgroup
     uint32_t *cand_cnt;        // append mode: [nq_tile][seg_stride] counts (above kSegCap: that segment overflowed)
     uint32_t seg_stride;       // segments allocated per query (>= grid of the launch)
+    uint32_t vgrid;            // single-tile permute-dot scan: four-wave groups of the launch (set by its launcher)
     int best_of_block;         // all-queries-per-pass kernel: no floor, per scanned block and query the best allowed slot (kModeBest)
     const uint32_t *run_if;    // append mode: when given and *run_if == 0 the launch does nothing (a level's conditional repeat)
 };

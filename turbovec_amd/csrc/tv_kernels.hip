@@ -490,8 +490,8 @@ __device__ __forceinline__ void stage_to_lds(uint4 *dst, const uint4 *src, int n
     }
 }
 
-template <int U, int MODE, bool W_LDS>
-__global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
+template <int U, int MODE, bool W_LDS, int THREADS = kScanThreads>
+__global__ __launch_bounds__(THREADS) void k_scan_p4(ScanArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr bool LISTS = MODE == kModeLists, DUMP = MODE == kModeDump, BEST = MODE == kModeBest;
     constexpr bool APPEND = MODE == kModeAppend || BEST;     // both fill the candidate segments
@@ -500,23 +500,31 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
     uint8_t *sW = smem + kDecodeBytes;
     const size_t w_bytes = kDecodeBytes + (W_LDS ? size_t(nch) * 2048 : 0);
     float *ls = reinterpret_cast<float *>(smem + w_bytes);
-    uint32_t *li = reinterpret_cast<uint32_t *>(ls + (LISTS ? k * kScanThreads : 0));
-    int *stau = reinterpret_cast<int *>(li + (LISTS ? k * kScanThreads : 0));
+    uint32_t *li = reinterpret_cast<uint32_t *>(ls + (LISTS ? k * THREADS : 0));
+    int *stau = reinterpret_cast<int *>(li + (LISTS ? k * THREADS : 0));
     uint32_t *scnt = reinterpret_cast<uint32_t *>(stau);  // append mode: candidates per query of this workgroup
 
+    // A workgroup of more than four waves is GROUPS four-wave groups that share the weights in LDS
+    // and are, in every other respect, workgroups vb of a launch of a.vgrid four-wave workgroups:
+    // the same blocks per wave, a candidate segment per group.
+    constexpr int GROUPS = THREADS / kScanThreads;
+    static_assert(THREADS % kScanThreads == 0 && (GROUPS == 1 || APPEND), "wave groups are an append-mode form");
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = (tid >> 6) % (kScanThreads / 64);
     const int qn = lane & 31, h = lane >> 5;
+    const uint32_t vgrid = GROUPS > 1 ? a.vgrid : gridDim.x;
+    const uint32_t vb = GROUPS > 1 ? blockIdx.x * GROUPS + uint32_t(tid) / kScanThreads : blockIdx.x;
+    if (GROUPS > 1) scnt += (tid / kScanThreads) * kQTile;
 
     // Logical blocks j = 0..nj-1 stand for physical blocks j*step (step > 1 samples the index).
     const uint32_t step = a.b_step;
     const uint32_t nj = (a.n_blocks + step - 1) / step;
-    const uint32_t total_waves = gridDim.x * (kScanThreads / 64);
-    const uint32_t gw = wave * gridDim.x + blockIdx.x;  // consecutive blocks go to different workgroups
+    const uint32_t total_waves = vgrid * (kScanThreads / 64);
+    const uint32_t gw = wave * vgrid + vb;  // consecutive blocks go to different workgroups
     // Blocks are dealt round-robin to the waves of the grid: wave gw takes logical blocks gw,
     // gw + total_waves, ...  Neighbouring rows (clustered data, contiguous allowlists) then spread
     // over all workgroups instead of piling into one.
-    const uint32_t j_begin = gw, j_end = nj;
+    const uint32_t j_begin = gw, j_end = (GROUPS > 1 && vb >= vgrid) ? 0u : nj;   // (a group beyond the launch's last has no blocks)
     const uint4 *codes = reinterpret_cast<const uint4 *>(a.codes) + lane;
 
     // first block with at least one allowed slot (search.rs:3015-3029)
@@ -539,14 +547,14 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
         for (int u = 0; u < U; ++u) buf[u] = load_stream16(&codes[(size_t(j) * step * nch + u) * 64]);
     }
 
-    if (W_LDS) stage_to_lds<kScanThreads>(reinterpret_cast<uint4 *>(sW), reinterpret_cast<const uint4 *>(a.tables), nch * 128, tid);
-    for (int b = tid; b < 256; b += kScanThreads) {
+    if (W_LDS) stage_to_lds<THREADS>(reinterpret_cast<uint4 *>(sW), reinterpret_cast<const uint4 *>(a.tables), nch * 128, tid);
+    for (int b = tid; b < 256; b += THREADS) {
         const uint32_t lo = (a.lv[(b & 15) >> 2] >> (8 * (b & 3))) & 0xffu;
         const uint32_t hi = (a.lv[b >> 6] >> (8 * ((b >> 4) & 3))) & 0xffu;
         reinterpret_cast<uint16_t *>(smem)[b] = uint16_t(lo | (hi << 8));
     }
     if (LISTS && tid < kQTile) stau[tid] = a.gtau[tid];
-    if (APPEND && tid < kQTile) scnt[tid] = 0u;
+    if (APPEND && (tid % kScanThreads) < kQTile) scnt[tid % kScanThreads] = 0u;
     __syncthreads();
 
     const bool active = qn < a.nq_tile;
@@ -667,7 +675,7 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
             if (oslot != 0xffffffffu && (bslot == 0xffffffffu || ranks_before(os_, oslot, bs, bslot))) { bs = os_; bslot = oslot; }
             if (h == 0 && bslot != 0xffffffffu) {
                 const uint32_t pos = atomicAdd(&scnt[qn], 1u);
-                if (pos < kSegCap) a.cand[(size_t(qn) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(bs, bslot);
+                if (pos < kSegCap) a.cand[(size_t(qn) * a.seg_stride + vb) * kSegCap + pos] = sort_key(bs, bslot);
             }
         } else if (APPEND) {
 #pragma unroll
@@ -679,7 +687,7 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
                     if (slot < a.n && ((mw >> i) & 1u)) {
                         const uint32_t pos = atomicAdd(&scnt[qn], 1u);
                         if (pos < kSegCap)
-                            a.cand[(size_t(qn) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(s, slot);
+                            a.cand[(size_t(qn) * a.seg_stride + vb) * kSegCap + pos] = sort_key(s, slot);
                     }
                 }
             }
@@ -693,7 +701,7 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
                 const float s = fmaf(float(acc[r]), qs, qb) * vs[r];
                 if (active && s >= tau && (L.cnt < k || ranks_before(s, slot, L.worst_s, L.worst_i))) {
                     if (slot < a.n && ((mw >> i) & 1u)) {
-                        if (list_offer(L, ls, li, kScanThreads, tid, k, s, slot) && a.share_tau) {
+                        if (list_offer(L, ls, li, THREADS, tid, k, s, slot) && a.share_tau) {
                             const int key = order_key(L.worst_s);
                             if (atomicMax(&stau[qn], key) < key) atomicMax(&a.gtau[qn], key);
                         }
@@ -705,17 +713,18 @@ __global__ __launch_bounds__(kScanThreads) void k_scan_p4(ScanArgs a) {
     }
 
     if (LISTS) {
-        const size_t total_threads = size_t(gridDim.x) * kScanThreads;
-        const size_t gt = size_t(blockIdx.x) * kScanThreads + tid;
+        const size_t total_threads = size_t(gridDim.x) * THREADS;
+        const size_t gt = size_t(blockIdx.x) * THREADS + tid;
         a.part_cnt[gt] = L.cnt;
         for (int e = 0; e < L.cnt; ++e) {
-            a.part_scores[size_t(e) * total_threads + gt] = ls[e * kScanThreads + tid];
-            a.part_idx[size_t(e) * total_threads + gt] = li[e * kScanThreads + tid];
+            a.part_scores[size_t(e) * total_threads + gt] = ls[e * THREADS + tid];
+            a.part_idx[size_t(e) * total_threads + gt] = li[e * THREADS + tid];
         }
     }
     if (APPEND) {
         __syncthreads();
-        if (tid < a.nq_tile) a.cand_cnt[size_t(tid) * a.seg_stride + blockIdx.x] = scnt[tid];
+        const int t = tid % kScanThreads;
+        if (t < a.nq_tile && vb < vgrid) a.cand_cnt[size_t(t) * a.seg_stride + vb] = scnt[t];
     }
 }
 
@@ -1671,35 +1680,65 @@ size_t scan_lds_bytes(int mode_p, int nch, int k, int lut_queries) {
     return size_t(nch) * 1024 * lut_queries + lists;
 }
 
+// Workgroup size of the append-mode permute-dot scan (sample-then-filter, up to 32 queries).  The
+// scan streams fastest with sixteen waves per CU on ONE copy of the query tile's weights in LDS:
+// a 1024-thread workgroup of four four-wave groups, each group with a candidate segment of its own
+// (the selection kernel reads short segments fastest).  Four-wave workgroups with a copy each (48 KiB
+// at 1536 dimensions) reach twelve waves per CU where three copies fit -- one query over 10M x 1536
+// bytes of codes at 128 to 1792 dimensions: 0.61-0.93 ms, the large workgroup 0.60-0.91, up to 18 %
+// less -- and four waves per CU from 2560 dimensions (0.88 ms against 0.60).  Rows whose weights do
+// not fit LDS (beyond 5056 dimensions) read them from global memory in four-wave workgroups.
+constexpr int kScanThreadsShared = 4 * kScanThreads;
+static int scan_p4_append_threads(int nch) {
+    const size_t lds = size_t(nch) * 2048 + kDecodeBytes + (kScanThreadsShared / kScanThreads) * kQTile * sizeof(int);
+    return lds <= kLdsBudget ? kScanThreadsShared : kScanThreads;
+}
+
 int scan_grid_blocks(int device, int mode_p, int nch, int k, int nq_tile) {
     hipDeviceProp_t prop;
     int cus = 256;
     if (hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0)
         cus = prop.multiProcessorCount;
+    if (mode_p && k == 0 && scan_p4_append_threads(nch) != kScanThreads)           // (k = 0: the append-mode scans)
+        return cus * (kScanThreadsShared / kScanThreads);                         // one workgroup per CU, counted in four-wave groups
     const size_t lds = scan_lds_bytes(mode_p, nch, k, nq_tile);
     int per_cu = int(kLdsBudget / (lds ? lds : 1));
     if (per_cu < 1) per_cu = 1;
     if (per_cu > 4) per_cu = 4;
+    // (the instances that read four or eight chunks per burst hold three waves per SIMD: a fourth
+    // workgroup per CU would only wait for a place and run as a tail)
+    if (mode_p && k == 0 && nch % 4 == 0 && per_cu > 3) per_cu = 3;
     return cus * per_cu;
 }
 
-hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s) {
+hipError_t launch_scan_p4(const ScanArgs &args, int grid, int mode, hipStream_t s) {
+    ScanArgs a = args;
+    const int threads = (mode == kModeAppend || mode == kModeBest) ? scan_p4_append_threads(a.nch) : kScanThreads;
+    const int groups = threads / kScanThreads;
+    a.vgrid = uint32_t(grid);                        // `grid` counts four-wave groups
+    const int wgs = (grid + groups - 1) / groups;
     const size_t w = size_t(a.nch) * 2048;
-    const size_t lists = kDecodeBytes + kQTile * sizeof(int) + (mode != kModeLists ? 0 : size_t(a.k) * kScanThreads * 8);
+    const size_t lists = kDecodeBytes + groups * kQTile * sizeof(int) + (mode != kModeLists ? 0 : size_t(a.k) * kScanThreads * 8);
     const bool w_lds = w + lists <= kLdsBudget;
     const size_t lds = (w_lds ? w : 0) + lists;
+    // (append-mode scans whose weights fit LDS take the large workgroup; four-wave ones read them from global memory)
+    if ((mode == kModeAppend || mode == kModeBest) && groups == 1 && w_lds) return hipErrorInvalidValue;
     hipError_t e = hipSuccess;
-#define TV_LAUNCH_P4(U, D, W)                                                                   \
+#define TV_LAUNCH_P4_T(U, D, W, T)                                                              \
     do {                                                                                        \
-        e = allow_lds(k_scan_p4<U, D, W>, lds);                                                 \
+        e = allow_lds(k_scan_p4<U, D, W, T>, lds);                                              \
         if (e != hipSuccess) return e;                                                          \
-        hipLaunchKernelGGL((k_scan_p4<U, D, W>), dim3(grid), dim3(kScanThreads), lds, s, a);    \
+        hipLaunchKernelGGL((k_scan_p4<U, D, W, T>), dim3(wgs), dim3(T), lds, s, a);             \
     } while (0)
+#define TV_LAUNCH_P4(U, D, W) TV_LAUNCH_P4_T(U, D, W, kScanThreads)
+// (sixteen waves per CU leave a wave 128 registers: the large workgroup reads bursts of four chunks
+// at most, and its floorless level -- a short launch either way -- of two)
 #define TV_PICK_P4(U)                                                                           \
     do {                                                                                        \
-        if (mode == kModeDump) { if (w_lds) TV_LAUNCH_P4(U, kModeDump, true); else TV_LAUNCH_P4(U, kModeDump, false); } \
-        else if (mode == kModeAppend) { if (w_lds) TV_LAUNCH_P4(U, kModeAppend, true); else TV_LAUNCH_P4(U, kModeAppend, false); } \
-        else if (mode == kModeBest) { if (w_lds) TV_LAUNCH_P4(U, kModeBest, true); else TV_LAUNCH_P4(U, kModeBest, false); } \
+        if (groups > 1) { if (mode == kModeAppend) TV_LAUNCH_P4_T((U > 4 ? 4 : U), kModeAppend, true, kScanThreadsShared); else TV_LAUNCH_P4_T((U > 2 ? 2 : U), kModeBest, true, kScanThreadsShared); } \
+        else if (mode == kModeDump) { if (w_lds) TV_LAUNCH_P4(U, kModeDump, true); else TV_LAUNCH_P4(U, kModeDump, false); } \
+        else if (mode == kModeAppend) TV_LAUNCH_P4(U, kModeAppend, false);                      \
+        else if (mode == kModeBest) TV_LAUNCH_P4(U, kModeBest, false);                          \
         else { if (w_lds) TV_LAUNCH_P4(U, kModeLists, true); else TV_LAUNCH_P4(U, kModeLists, false); } \
     } while (0)
     if (a.nch % 8 == 0) TV_PICK_P4(8);          // 8 KiB per wave in flight: +3 % over 4 at 24 chunks, 12 is slower
@@ -1708,6 +1747,7 @@ hipError_t launch_scan_p4(const ScanArgs &a, int grid, int mode, hipStream_t s) 
     else TV_PICK_P4(1);
 #undef TV_PICK_P4
 #undef TV_LAUNCH_P4
+#undef TV_LAUNCH_P4_T
     return hipGetLastError();
 }
 
