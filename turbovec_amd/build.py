@@ -31,9 +31,11 @@ FLAGS = [
 # (k_scan_p4, k_scan_p4_multi, k_scan_p4_wide, k_scan_lut16 and the matrix-unit probe;
 # k_scan_p4_batched and the other LUT scans leave every wait to the compiler.)
 NO_SCRATCH = re.compile(r"k_scan_p4I|k_scan_p4_multiI|k_scan_p4_wideI|k_scan_lut16I|k_probe_mfma")
-# These two address their byte -> levels table by the byte's value alone: the table must sit at LDS
-# address 0, i.e. the kernel may have no static LDS allocation in front of its dynamic one.
-NO_STATIC_LDS = re.compile(r"k_scan_p4(_multi)?I")
+# These address their byte -> levels table by the byte's value alone: the table must sit at LDS
+# address 0, i.e. the kernel may have no static LDS allocation in front of its dynamic one
+# (k_scan_p4, k_scan_p4_multi, and the instances of k_scan_p4_wide whose last template argument,
+# the split decode, is true).
+NO_STATIC_LDS = re.compile(r"k_scan_p4(_multi)?I|k_scan_p4_wideI.*Lb1EEEv")
 
 
 def check_resources(src, remarks):

@@ -666,7 +666,7 @@ int search_device(tv_index *ix, const float *d_queries, size_t nq, size_t k, con
             Prepared pq;
             const int nt_batched = plan.nt_batched;
             int prc = prepare_queries(ix, ar, repeat ? d_redo_q : d_q, pq_n, pq,
-                                      !wide && (nt_batched == 0 || tv::batched_weights_split(g.nch)), false, true);
+                                      wide ? tv::wide_weights_split(g.nch) : (nt_batched == 0 || tv::batched_weights_split(g.nch)), false, true);
             if (prc != TV_OK) return prc;
             uint64_t *d_cand = ar.take<uint64_t>(cq_pad * seg_stride * tv::kSegCap);
             uint32_t *d_cnt = ar.take<uint32_t>(cq_pad * seg_stride);

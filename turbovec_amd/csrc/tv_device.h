@@ -131,6 +131,27 @@ __device__ __forceinline__ uint32_t levels_of(uint32_t nib, uint32_t t0, uint32_
     return __builtin_amdgcn_perm(t1, t0, selA) & __builtin_amdgcn_perm(t3, t2, selB);
 }
 
+// The code byte -> (level of its low nibble, level of its high nibble) table the permute-dot scans
+// keep at the start of their LDS: 256 entries of two int8 levels.
+constexpr int kDecodeBytes = 512;
+
+// A 16-bit LDS load, zero-extended, requested without telling the compiler's wait-count
+// bookkeeping (the caller's `s_waitcnt lgkmcnt(N)`, tied to the destinations, is the matching
+// wait).  The loads that fill one half of a register and keep the other are no use here: with
+// ECC-protected register files they clear it.
+__device__ __forceinline__ void lds_u16(uint32_t &dst, uint32_t addr) {
+    asm volatile("ds_read_u16 %0, %1" : "=v"(dst) : "v"(addr));
+}
+// 2 * byte E of x: the offset of that code byte's table entry.
+template <int E>
+__device__ __forceinline__ uint32_t byte_x2(uint32_t x) {
+    uint32_t r;
+    if (E == 0) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0" : "=v"(r) : "v"(1u), "v"(x));
+    if (E == 1) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1" : "=v"(r) : "v"(1u), "v"(x));
+    if (E == 2) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2" : "=v"(r) : "v"(1u), "v"(x));
+    if (E == 3) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3" : "=v"(r) : "v"(1u), "v"(x));
+    return r;
+}
 
 // A conditional launch: true when the flag it depends on says there is nothing to do.  The flag is
 // uniform over the grid and written by an earlier launch of the same stream.

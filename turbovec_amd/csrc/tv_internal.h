@@ -137,6 +137,7 @@ hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s);
 int wide_blocks_per_workgroup(int nch);
 bool wide_serves_best_of_block(int nch);
 int wide_max_queries(int nch);
+bool wide_weights_split(int nch);
 
 hipError_t launch_merge(const float *part_scores, const uint32_t *part_idx, const int *part_cnt, int total_threads,
                         int qmod, int k, int k_eff, int nq_tile, float *out_scores, int64_t *out_idx,

@@ -429,25 +429,8 @@ __global__ __launch_bounds__(256) void k_build_lut(const float *__restrict__ qca
 // The table sits at the start of the kernel's LDS (there is no static
 // allocation before it), so a byte's offset is its address.
 // ===========================================================================
-constexpr int kDecodeBytes = 512;
-
-// A 16-bit LDS load, zero-extended, requested without telling the compiler's wait-count
-// bookkeeping (lds_settle is the matching wait).  The loads that fill one half of a register
-// and keep the other are no use here: with ECC-protected register files they clear it.
-__device__ __forceinline__ void lds_u16(uint32_t &dst, uint32_t addr) {
-    asm volatile("ds_read_u16 %0, %1" : "=v"(dst) : "v"(addr));
-}
-// 2 * byte E of x: the offset of that code byte's table entry.
-template <int E>
-__device__ __forceinline__ uint32_t byte_x2(uint32_t x) {
-    uint32_t r;
-    if (E == 0) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0" : "=v"(r) : "v"(1u), "v"(x));
-    if (E == 1) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1" : "=v"(r) : "v"(1u), "v"(x));
-    if (E == 2) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2" : "=v"(r) : "v"(1u), "v"(x));
-    if (E == 3) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3" : "=v"(r) : "v"(1u), "v"(x));
-    return r;
-}
-// 16 bytes of LDS per lane, requested the same way.
+// 16 bytes of LDS per lane, requested like the table entries (lds_u16): behind the compiler's
+// wait-count bookkeeping, lds_settle being the matching wait.
 template <int OFF>
 __device__ __forceinline__ void lds_b128(v4i &dst, uint32_t addr) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(dst) : "v"(addr), "n"(OFF));

@@ -97,6 +97,7 @@ struct WideQueryTail {
     uint32_t cnt;           // candidates this workgroup appended
 };
 constexpr int kWideQueryBytes = int(sizeof(WideQuery) + sizeof(WideQueryTail));
+constexpr int kWideTableBytes = 1024;    // the byte table of the split decode (kDecodeBytes), padded to the ring's alignment
 
 // WAVES = 8 (two per SIMD, 256 VGPRs each) holds rows of up to 24 chunks; WAVES = 4 (one per SIMD)
 // gives a wave the whole 512-register file -- the compiler keeps what does not fit the VGPRs in
@@ -111,14 +112,24 @@ constexpr int kWideQueryBytes = int(sizeof(WideQuery) + sizeof(WideQueryTail));
 // end of a tile the odd wave hands its partial sums to the even one through LDS, which adds them
 // and does the tile's bound test and scoring.  Two blocks per workgroup instead of four, one more
 // barrier per tile: the form for rows beyond what one wave holds.
-template <int NCH, int NB, int WAVES, int SPT, int BLK, int HO, int KS>
+//
+// SPLIT: the block phase decodes half of every chunk through the byte table in LDS, like
+// k_scan_p4 (code bytes 0-7 of a lane on the vector ALU, bytes 8-15 looked up whole); the weights
+// then come in that kernel's split order.  The decode is the block phase -- both waves of a SIMD
+// at it together, the matrix unit idle -- and the LDS has nothing else to do then.
+template <int NCH, int NB, int WAVES, int SPT, int BLK, int HO, int KS, bool SPLIT = false>
 __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide(ScanArgs a) {
     static_assert(NCH % SPT == 0, "a slice is a whole number of chunks");
+    static_assert(!SPLIT || (WAVES == 8 && BLK == 1 && KS == 1), "the split decode is built for the one-block eight-wave forms");
     static_assert(KS == 1 || (KS == 2 && WAVES == 4 && BLK == 1 && HO == 1), "row halves go to the wave pairs of the four-wave form");
     constexpr int kWideRing = wide_ring(HO);
     static_assert(HO == 1 || (SPT % HO == 0 && kWideRing >= 2 * HO + 1), "slices handed over together must fit the ring twice");
-    extern __shared__ __align__(16) uint8_t smem[];
+    extern __shared__ __align__(16) uint8_t smem_all[];
     if (launch_switched_off(a.run_if)) return;
+    // (the byte table, when there is one, sits at the start of the kernel's LDS -- no static
+    // allocation precedes it -- so that a code byte's offset in it is its address)
+    // (... and the slice ring behind it keeps the 1 KiB alignment of its direct-to-LDS loads)
+    uint8_t *smem = smem_all + (SPLIT ? kWideTableBytes : 0);
     constexpr int kWideThreads = WAVES * 64, kWideWaves = WAVES;
     constexpr int kSC = NCH / SPT;                          // chunks per slice
     constexpr int kM = 2 * kSC;                             // MFMAs per wave and slice: (low, high) of each chunk
@@ -169,7 +180,14 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
         sq[q].ta = !act ? inf : bounded ? (tau / qs) * (1.0f - 1e-5f) : -inf;
         sq[q].tb = act && bounded ? rb + 1e-5f * fabsf(rb) + 2.0f : 0.0f;
     }
-    if (tid == 0) { snext[0] = 0u; snext[1] = 0u; }
+    if constexpr (SPLIT) {
+        for (int b = tid; b < 256; b += kWideThreads) {
+            const uint32_t lo = (a.lv[(b & 15) >> 2] >> (8 * (b & 3))) & 0xffu;
+            const uint32_t hi = (a.lv[b >> 6] >> (8 * ((b >> 4) & 3))) & 0xffu;
+            reinterpret_cast<uint16_t *>(smem_all)[b] = uint16_t(lo | (hi << 8));
+        }
+    }
+    if (tid == 0) { snext[0] = 0u; snext[1] = 0u; snext[2] = 0u; snext[3] = 0u; snext[4] = 0u; }
     uint32_t *s_over = snext + 1;                           // queries whose segment of this workgroup is full
     __syncthreads();
 
@@ -305,6 +323,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     int inv_vmax[BLK];       // bits of 1 / (largest allowed row scale of the block); +inf when that is 0
     bool odd_block[BLK];
     uint32_t blk[BLK];       // the wave's blocks of this round
+    uint32_t round_no = 0;
     for (;;) {
         // ---- block phase: claim, load, decode into registers ----
         bool has = false;
@@ -340,14 +359,57 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
                     constexpr int c = (decltype(ii)::value + kFirst) % NCH;
                     load16_async_s(raw[c], p + size_t(c) * 1024, lane16);
                 });
+                uint32_t te[2][4], to[2][4];    // (split decode) table entries on their way, this chunk's and the next's
                 static_for<NCH>([&](auto ii) {
                     constexpr int c = (decltype(ii)::value + kFirst) % NCH;
                     wait_vm<NCH - 1 - decltype(ii)::value>(raw[c]);
                     const uint32_t x[4] = {raw[c].x, raw[c].y, raw[c].z, raw[c].w};
+                    if constexpr (SPLIT) {
+                        // the chunk's first operand from code bytes 0..7 on the vector ALU (low-nibble
+                        // levels of bytes 0..3, high-nibble levels of bytes 0..3, the same of 4..7), the
+                        // second from bytes 8..15 through the table: dword r = entries of bytes 8+2r
+                        // and 9+2r.  The next chunk's entries are requested before this chunk's are
+                        // waited for, so that the LDS answers while the ALU works.  No other LDS or
+                        // scalar-memory request of this wave is in flight here (the B stream is
+                        // closed, the claim has returned), so the counts are exact.
+                        constexpr int i = decltype(ii)::value, p = i & 1;
+                        auto request = [&](auto cc, auto pp) {
+                            constexpr int cn = decltype(cc)::value, pn = decltype(pp)::value;
+                            const uint32_t xa = raw[cn].z, xb = raw[cn].w;
+                            lds_u16(te[pn][0], byte_x2<0>(xa)); lds_u16(to[pn][0], byte_x2<1>(xa));
+                            lds_u16(te[pn][1], byte_x2<2>(xa)); lds_u16(to[pn][1], byte_x2<3>(xa));
+                            lds_u16(te[pn][2], byte_x2<0>(xb)); lds_u16(to[pn][2], byte_x2<1>(xb));
+                            lds_u16(te[pn][3], byte_x2<2>(xb)); lds_u16(to[pn][3], byte_x2<3>(xb));
+                        };
+                        if constexpr (i == 0) request(IntC<c>{}, IntC<p>{});
+                        if constexpr (i + 1 < NCH) {
+                            constexpr int cn = (i + 1 + kFirst) % NCH;
+                            wait_vm<NCH - 2 - i>(raw[cn]);
+                            request(IntC<cn>{}, IntC<1 - p>{});
+                        }
+                        alo[k][c][0] = int(levels_of(x[0] & 0x0f0f0f0fu, t0, t1, t2, t3));
+                        alo[k][c][1] = int(levels_of((x[0] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
+                        alo[k][c][2] = int(levels_of(x[1] & 0x0f0f0f0fu, t0, t1, t2, t3));
+                        alo[k][c][3] = int(levels_of((x[1] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
+                        if constexpr (i + 1 < NCH)
+                            asm volatile("s_waitcnt lgkmcnt(8)"
+                                         : "+v"(te[p][0]), "+v"(te[p][1]), "+v"(te[p][2]), "+v"(te[p][3]), "+v"(to[p][0]), "+v"(to[p][1]), "+v"(to[p][2]), "+v"(to[p][3])
+                                         :: "memory");
+                        else
+                            asm volatile("s_waitcnt lgkmcnt(0)"
+                                         : "+v"(te[p][0]), "+v"(te[p][1]), "+v"(te[p][2]), "+v"(te[p][3]), "+v"(to[p][0]), "+v"(to[p][1]), "+v"(to[p][2]), "+v"(to[p][3])
+                                         :: "memory");
 #pragma unroll
-                    for (int d = 0; d < 4; ++d) {
-                        alo[k][c][d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
-                        ahi[k][c][d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
+                        for (int d = 0; d < 4; ++d) ahi[k][c][d] = int(te[p][d] | (to[p][d] << 16));
+                        // one chunk after the other: left to itself the scheduler works on several at
+                        // once and runs out of registers
+                        asm volatile("" : "+v"(alo[k][c]), "+v"(ahi[k][c]));
+                    } else {
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            alo[k][c][d] = int(levels_of(x[d] & 0x0f0f0f0fu, t0, t1, t2, t3));
+                            ahi[k][c][d] = int(levels_of((x[d] >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3));
+                        }
                     }
                     if constexpr (kHandMfma && c >= kVecChunks) {
                         // into its accumulation registers now, not at the first MFMA that reads it
@@ -377,7 +439,21 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
             odd_block[k] = __any(odd) || (vmax > 0.0f && vmax < 1e-30f);
             inv_vmax[k] = __builtin_amdgcn_readfirstlane(__float_as_int(inv));
         });
-        if (!__syncthreads_or(has ? 1 : 0)) break;
+        if constexpr (SPLIT) {
+            // "does any wave have a block?" through three rotating LDS flags instead of
+            // __syncthreads_or, whose static LDS word would sit in front of the byte table: round r
+            // sets and reads flag r % 3 on either side of the barrier and clears the next round's,
+            // which every wave has finished reading (two barriers ago).
+            uint32_t *flag = snext + 2;
+            if (tid == 0) flag[(round_no + 1) % 3u] = 0u;
+            if (has && lane == 0) flag[round_no % 3u] = 1u;
+            __syncthreads();
+            const bool any = __builtin_amdgcn_readfirstlane(int(*reinterpret_cast<volatile uint32_t *>(&flag[round_no % 3u]))) != 0;   // (uniform, and known to be)
+            ++round_no;
+            if (!any) break;
+        } else {
+            if (!__syncthreads_or(has ? 1 : 0)) break;
+        }
 
         // ---- tile phase ----
         // Scores of tile t for block k of this wave; lane owns query t*32 + qn and rows
@@ -590,15 +666,15 @@ int wide_blocks_per_workgroup(int nch) {
     }
 }
 
-static size_t wide_lds_bytes(int ring, int slot_bytes, int nq, int blk, int ks) {
+static size_t wide_lds_bytes(int ring, int slot_bytes, int nq, int blk, int ks, bool split = false) {
     const size_t nq_pad = size_t((nq + kQTile - 1) / kQTile) * kQTile;
     return size_t(ring) * slot_bytes + nq_pad * kWideQueryBytes + size_t(kWideWaves) * blk * 32 * 4 + 64 +
-           (ks == 2 ? 2 * 4096 : 0);
+           (ks == 2 ? 2 * 4096 : 0) + (split ? kWideTableBytes : 0);
 }
 
 // Most queries (whole tiles) a launch with this ring fits into the 160 KiB of LDS.
-static int wide_max_queries_of(int ring, int slot_bytes, int blk, int ks) {
-    const size_t fixed = wide_lds_bytes(ring, slot_bytes, 0, blk, ks);
+static int wide_max_queries_of(int ring, int slot_bytes, int blk, int ks, bool split = false) {
+    const size_t fixed = wide_lds_bytes(ring, slot_bytes, 0, blk, ks, split);
     if (fixed >= 160 * 1024) return 0;
     return int((160 * 1024 - fixed) / kWideQueryBytes / kQTile * kQTile);
 }
@@ -607,7 +683,7 @@ static int wide_max_queries_of(int ring, int slot_bytes, int blk, int ks) {
 // 1024 wherever there is one.
 int wide_max_queries(int nch) {
     switch (nch) {
-        case 24: return std::min(2048, wide_max_queries_of(wide_ring(4), 12 * 1024, 1, 1));
+        case 24: return std::min(2048, wide_max_queries_of(wide_ring(4), 12 * 1024, 1, 1, wide_weights_split(24)));
         default: return wide_blocks_per_workgroup(nch) > 0 ? 1024 : 0;
     }
 }
@@ -620,18 +696,22 @@ int wide_grid_blocks(int device) {
     return cus;      // one 8-wave workgroup per CU: its LDS holds the slice ring
 }
 
-template <int NCH, int NB, int WAVES = 8, int SPT = 2, int BLK = 1, int HO = 1, int KS = 1>
+template <int NCH, int NB, int WAVES = 8, int SPT = 2, int BLK = 1, int HO = 1, int KS = 1, bool SPLIT = false>
 static hipError_t launch_wide_n(const ScanArgs &a, int grid, hipStream_t s) {
-    const size_t lds = wide_lds_bytes(wide_ring(HO), KS * 2 * (NCH / SPT) * 1024, a.nq_tile, BLK, KS);
+    const size_t lds = wide_lds_bytes(wide_ring(HO), KS * 2 * (NCH / SPT) * 1024, a.nq_tile, BLK, KS, SPLIT);
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK, HO, KS>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK, HO, KS, SPLIT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK, HO, KS>), dim3(grid), dim3(WAVES * 64), lds, s, a);
+    hipLaunchKernelGGL((k_scan_p4_wide<NCH, NB, WAVES, SPT, BLK, HO, KS, SPLIT>), dim3(grid), dim3(WAVES * 64), lds, s, a);
     return hipGetLastError();
 }
+
+// Row lengths whose instance decodes half of a chunk through the LDS byte table: their weights
+// come in the split order of k_scan_p4 (launch_build_p / launch_prep_p, `split`).
+bool wide_weights_split(int nch) { return nch >= 12 && nch <= 24; }
 
 // a.nq_tile = all queries of the launch (any number up to the chunk size), a.tables = their
 // ceil(nq/32) weight tiles back to back, a.qscale / a.qbias / a.gtau indexed by query.
@@ -645,18 +725,18 @@ hipError_t launch_scan_p4_wide(const ScanArgs &a, int grid, hipStream_t s) {
         case 6: return launch_wide_n<6, 2, 8, 1, 3>(a, grid, s);
         case 8: return launch_wide_n<8, 4, 8, 1, 2>(a, grid, s);
         case 10: return launch_wide_n<10, 2, 8, 2, 2, 2>(a, grid, s);
-        case 12: return launch_wide_n<12, 2, 8, 2, 1, 2>(a, grid, s);   // two blocks per wave would spill 21 registers
-        case 14: return launch_wide_n<14, 2, 8, 2, 1, 2>(a, grid, s);
-        case 16: return launch_wide_n<16, 4, 8, 2, 1, 2>(a, grid, s);
-        case 18: return launch_wide_n<18, 2, 8, 2, 1, 2>(a, grid, s);
-        case 20: return launch_wide_n<20, 2, 8, 2, 1, 2>(a, grid, s);   // (four operand registers in flight would spill one)
-        case 22: return launch_wide_n<22, 2, 8, 2, 1, 2>(a, grid, s);
+        case 12: return launch_wide_n<12, 2, 8, 2, 1, 2, 1, true>(a, grid, s);   // two blocks per wave would spill 21 registers
+        case 14: return launch_wide_n<14, 2, 8, 2, 1, 2, 1, true>(a, grid, s);
+        case 16: return launch_wide_n<16, 4, 8, 2, 1, 2, 1, true>(a, grid, s);
+        case 18: return launch_wide_n<18, 2, 8, 2, 1, 2, 1, true>(a, grid, s);
+        case 20: return launch_wide_n<20, 2, 8, 2, 1, 2, 1, true>(a, grid, s);   // (four operand registers in flight would spill one)
+        case 22: return launch_wide_n<22, 2, 8, 2, 1, 2, 1, true>(a, grid, s);
         // 24 chunks (1536 dimensions): up to 1632 queries with the ring of five 24 KiB slices; longer
         // chunks (to 2048 queries: a block is then decoded once per 64 tiles instead of 32) with a
         // ring of nine 12 KiB slices handed over four at a time, which leaves the LDS for them
         case 24:
-            if (a.nq_tile <= wide_max_queries_of(wide_ring(2), 24 * 1024, 1, 1)) return launch_wide_n<24, 2, 8, 2, 1, 2>(a, grid, s);
-            return launch_wide_n<24, 2, 8, 4, 1, 4>(a, grid, s);
+            if (a.nq_tile <= wide_max_queries_of(wide_ring(2), 24 * 1024, 1, 1, true)) return launch_wide_n<24, 2, 8, 2, 1, 2, 1, true>(a, grid, s);
+            return launch_wide_n<24, 2, 8, 4, 1, 4, 1, true>(a, grid, s);
         case 28: return launch_wide_n<28, 2, 4, 4, 1>(a, grid, s);
         case 32: return launch_wide_n<32, 4, 4, 4, 1>(a, grid, s);
         case 36: return launch_wide_n<36, 2, 4, 4, 1>(a, grid, s);
