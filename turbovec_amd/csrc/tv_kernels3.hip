@@ -49,6 +49,11 @@ __device__ __forceinline__ void load16_async_s(u32x4 &dst, const void *sbase, ui
     asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(dst) : "v"(lane16), "s"(sbase));
 }
 
+// One word of LDS by its address, read afresh every time.
+__device__ __forceinline__ uint32_t lds_word(uint32_t addr) {
+    return *reinterpret_cast<const volatile __attribute__((address_space(3))) uint32_t *>(uintptr_t(addr));
+}
+
 // 16 bytes of LDS per lane, requested without telling the compiler's wait-count bookkeeping;
 // lds_wait<N> on the destination holds until at most N younger LDS requests are outstanding.
 template <int OFF>
@@ -189,6 +194,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
     }
     if (tid == 0) { snext[0] = 0u; snext[1] = 0u; snext[2] = 0u; snext[3] = 0u; snext[4] = 0u; }
     uint32_t *s_over = snext + 1;                           // queries whose segment of this workgroup is full
+    const uint32_t s_over_addr = lds_b + uint32_t(reinterpret_cast<uint8_t *>(s_over) - smem);
     __syncthreads();
 
     const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
@@ -336,7 +342,9 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
         // sits out would add stale partial sums -- so the pair form reads it behind a barrier every
         // wave's appends of the round before have passed.)
         if constexpr (KS == 2) __syncthreads();
-        const bool futile = uint32_t(__builtin_amdgcn_readfirstlane(int(*reinterpret_cast<volatile uint32_t *>(s_over)))) >= uint32_t(nq);
+        // (read as LDS, not through a generic pointer: a flat load is counted by both memory
+        // counters and the compiler would wait for every weight request in flight before it)
+        const bool futile = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_word(s_over_addr)))) >= uint32_t(nq);
         static_for<BLK>([&](auto kk) {
             constexpr int k = decltype(kk)::value;
             const uint32_t j = futile ? nj : claim();
@@ -448,7 +456,7 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 8 ? 2 : 1) void k_scan_p4_wide
             if (tid == 0) flag[(round_no + 1) % 3u] = 0u;
             if (has && lane == 0) flag[round_no % 3u] = 1u;
             __syncthreads();
-            const bool any = __builtin_amdgcn_readfirstlane(int(*reinterpret_cast<volatile uint32_t *>(&flag[round_no % 3u]))) != 0;   // (uniform, and known to be)
+            const bool any = __builtin_amdgcn_readfirstlane(int(lds_word(s_over_addr + 4u + 4u * (round_no % 3u)))) != 0;   // (uniform, and known to be)
             ++round_no;
             if (!any) break;
         } else {
