@@ -274,3 +274,47 @@ def test_paths_agree_on_random_shapes(T):
             assert np.array_equal(res[0][1], i) and bits_equal(res[0][0], s), (case, dim, n, nq, k, kind)
         ix.close()
         del v
+
+
+# the same for batches below the wide kernel's: the single-tile scan (one to 32 queries, every
+# burst length of its sixteen-wave form, rows whose weights do not fit LDS), the resident-weights
+# tile-group kernel (two to four tiles) and the streamed one (two to four tiles, from 2560
+# dimensions) against the exact full-list path, bit for bit
+def test_small_batches_agree_with_the_exact_path_on_random_shapes(T):
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(77)
+    dims = [128, 192, 256, 320, 384, 512, 704, 768, 1024, 1280, 1472, 1536, 1792, 2048, 2560, 2624, 3072, 4096, 5120, 5376]
+    for case in range(36):
+        dim = int(rng.choice(dims))
+        n = int(rng.integers(40, 90_000 if dim <= 1536 else 30_000))
+        nq = int(rng.choice([1, 2, 7, 8, 9, 16, 31, 32, 33, 45, 64, 65, 70, 96, 97, 128]))
+        k = int(rng.choice([1, 10, 16, 64, 100]))
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(case * 104729 + 3)
+        ix = T.NativeIndex(dim, 4)
+        v = torch.randn(n, dim, device=dev, generator=gen)
+        if rng.random() < 0.3:
+            v *= torch.exp(torch.randn(n, 1, device=dev, generator=gen))
+        if rng.random() < 0.2:
+            v[: n // 3] = v[n // 3: 2 * (n // 3)]
+        torch.cuda.synchronize()
+        ix.add_dev(v.data_ptr(), n)
+        q = torch.randn(nq, dim, device=dev, generator=gen).cpu().numpy()
+        kind = int(rng.integers(0, 4))
+        m = None
+        if kind == 1:
+            m = rng.random(n) < rng.choice([0.5, 0.05, 0.002])
+        elif kind == 2:
+            lo = int(rng.integers(0, n))
+            m = (np.arange(n) >= lo) & (np.arange(n) < lo + max(1, n // 20))
+        elif kind == 3:
+            m = np.zeros(n, bool)
+            m[rng.integers(0, n, size=min(n, 7))] = True
+        words = None if m is None else T.pack_mask(m)[0]
+        res = []
+        for path in (0, 1):
+            ix.set_path(path)
+            res.append(ix.search(q, k, mask_words=words))
+        assert np.array_equal(res[0][1], res[1][1]) and bits_equal(res[0][0], res[1][0]), (case, dim, n, nq, k, kind)
+        ix.close()
+        del v
