@@ -340,9 +340,9 @@ SampledPlan sampled_plan(const tv_index *ix, size_t cq) {
                     : tv::lut_append_grid(ix->device, g.nch);
     p.lut_single = !mode_p && cq == 1 && effective_mode(ix) != TV_SCORE_L_SCALAR && tv::lut_single_uses_byte_tables(g.nch, p.grid);
     p.seg_stride = size_t(p.grid);
-    // (a query keeps one candidate segment per workgroup of the largest launch that serves it: the
-    // tile-group kernels' grid is not the single-tile scan's, and on long rows it is the larger one)
-    if (p.nt_batched > 0 && !p.wide) p.seg_stride = std::max(p.seg_stride, size_t(tv::batched_grid_blocks(ix->device, g.nch)));
+    // (a query keeps one candidate segment per workgroup of the launches that serve it: every launch
+    // of a chunk the tile-group kernels serve is one of theirs, and their grid is not the single-tile scan's)
+    if (p.nt_batched > 0 && !p.wide) p.seg_stride = size_t(tv::batched_grid_blocks(ix->device, g.nch));
     p.need = prepare_bytes(ix, cq) + round_up(p.n_tiles * tv::kQTile * 4, 256) +
              round_up(p.cq_pad * p.seg_stride * tv::kSegCap * 8, 256) + round_up(p.cq_pad * p.seg_stride * 4, 256) +
              round_up(p.cq_pad * 4, 256) + 65536;
