@@ -65,7 +65,7 @@ struct ScanArgs {
     int n_groups;              // byte groups of a row that carry codes (the rest of the last chunks is padding)
     uint32_t b_step;           // 1, or a sampling stride: only blocks j*b_step are scanned
     int share_tau;             // lists mode: waves share and raise gtau while scanning
-    uint64_t *cand;            // append mode: [nq_tile][seg_stride][kSegCap] sort keys, one segment per workgroup
+    uint64_t *cand;            // append mode: [nq_tile][seg_stride][kSegCap] sort keys, one segment per workgroup (per four-wave group in the single-tile permute-dot scan)
     uint32_t *cand_cnt;        // append mode: [nq_tile][seg_stride] counts (above kSegCap: that segment overflowed)
     uint32_t seg_stride;       // segments allocated per query (>= grid of the launch)
     uint32_t vgrid;            // single-tile permute-dot scan: four-wave groups of the launch (set by its launcher)
