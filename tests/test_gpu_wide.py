@@ -318,3 +318,39 @@ def test_small_batches_agree_with_the_exact_path_on_random_shapes(T):
         assert np.array_equal(res[0][1], res[1][1]) and bits_equal(res[0][0], res[1][0]), (case, dim, n, nq, k, kind)
         ix.close()
         del v
+
+
+# the tile-group kernel tests the same accumulator bound before it scores a tile in floats
+@pytest.mark.parametrize("dim,nq", [(1536, 64), (1536, 96), (512, 128), (2048, 40)])
+def test_tile_group_scan_with_wild_row_scales_and_query_scales(T, oracle, dim, nq):
+    """Row scales far from the encoder's (zeros, tiny, huge, then negative ones mixed in) and queries
+    scaled by powers of two far outside the unit range (floors and query scales beyond the range the
+    bound is derived for switch it off) on batches the tile-group kernels serve: against the oracle,
+    and against the exact path."""
+    n = 5_003
+    oidx = OracleIndex(oracle, dim, 4, unit_gaussian(n, dim, seed=61))
+    rng = np.random.default_rng(62)
+    factors = rng.choice(np.array([0.0, 1e-12, 1e-3, 1.0, 3.7, 1e6], np.float32), size=n)
+    oidx.scales = (oidx.scales * factors).astype(np.float32)
+    q = unit_gaussian(nq, dim, seed=63)
+    ix = to_native(T, oidx)
+    for k in (1, 10, 100):
+        s, i = ix.search(q, k)
+        assert 32 < ix.queries_per_launch() <= 128
+        os_, oi = oidx.search(q, k)
+        assert np.array_equal(i, oi) and bits_equal(s, os_), k
+    for e in (-120, -60, 40, 100):
+        qe = q * np.float32(2.0 ** e)
+        s, i = ix.search(qe, 10)
+        os_, oi = oidx.search(qe, 10)
+        assert np.array_equal(i, oi) and bits_equal(s, os_), e
+    ix.close()
+    oidx.scales[rng.random(n) < 0.02] *= np.float32(-1.0)
+    ix = to_native(T, oidx)
+    for k in (10, 100):
+        s, i = ix.search(q, k)
+        ix.set_path(1)
+        s3, i3 = ix.search(q, k)
+        ix.set_path(0)
+        assert np.array_equal(i, i3) and bits_equal(s, s3), k
+    ix.close()

@@ -738,26 +738,32 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
         const uint32_t hi = (a.lv[b >> 6] >> (8 * ((b >> 4) & 3))) & 0xffu;
         reinterpret_cast<uint16_t *>(smem)[b] = uint16_t(lo | (hi << 8));
     }
-    for (int i = tid; i < NT * kQTile; i += THREADS) scnt[i] = 0u;
     uint32_t *snext = scnt + NT * kQTile;   // next unclaimed block of this workgroup
+    // Per query, in LDS (a block's epilogue reads them; registers are for the stream): scale, bias
+    // and floor, and the accumulator bound of k_scan_p4_wide -- a row reaches its query's floor only
+    // if its integer sum reaches  floor / (qscale * largest row scale of the block) - qbias / qscale,
+    // taken conservatively (1e-5 relative, 2 + 1 absolute), so a tile of a block is scored in
+    // floats only when some lane's largest sum is at the bound.  Floors, query scales and biases
+    // outside 1e-30 .. 1e30 switch the bound off for that query (every tile scored).
+    float4 *s_q = reinterpret_cast<float4 *>(snext + 4);      // [NT * 32] (scale, bias, floor, -)
+    float2 *s_b = reinterpret_cast<float2 *>(s_q + NT * kQTile);   // [NT * 32] (ta, tb) of the bound
+    for (int q = tid; q < NT * kQTile; q += THREADS) {
+        scnt[q] = 0u;
+        const bool act = q < a.nq_tile;
+        const float qs = act ? a.qscale[q] : 0.0f, qb = act ? a.qbias[q] : 0.0f;
+        const float tau = act ? order_unkey(a.gtau[q]) : __int_as_float(0x7fc00000);  // NaN: nothing passes
+        s_q[q] = make_float4(qs, qb, tau, 0.0f);
+        const float inf = __int_as_float(0x7f800000);
+        const bool bounded = tau >= 1e-30f && tau <= 1e30f && qs >= 1e-30f && qs <= 1e30f && fabsf(qb) <= 1e30f &&
+                             tau / qs < inf;
+        const float rb = qb / qs;
+        s_b[q] = make_float2(!act ? inf : bounded ? (tau / qs) * (1.0f - 1e-5f) : -inf,
+                             act && bounded ? rb + 1e-5f * fabsf(rb) + 2.0f : 0.0f);
+    }
     if (tid == 0) *snext = 0u;
     __syncthreads();
 
-    float qs[NT], qb[NT], tau[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        const int q = t * kQTile + qn;
-        const bool act = q < a.nq_tile;
-        qs[t] = act ? a.qscale[q] : 0.0f;
-        qb[t] = act ? a.qbias[q] : 0.0f;
-        tau[t] = act ? order_unkey(a.gtau[q]) : __int_as_float(0x7fc00000);  // NaN: nothing passes
-        // Pass the three through a register move the compiler cannot see through: it then waits
-        // for these loads here, once, instead of before their first use inside the stream, where
-        // a full wait would also drain the code loads in flight.
-        asm volatile("v_mov_b32 %0, %0\n v_mov_b32 %1, %1\n v_mov_b32 %2, %2" : "+v"(qs[t]), "+v"(qb[t]), "+v"(tau[t]));
-    }
     const uint32_t t0 = a.lv[0], t1 = a.lv[1], t2 = a.lv[2], t3 = a.lv[3];
-
     const uint32_t step = a.b_step;
     const uint32_t nj = (a.n_blocks + step - 1) / step;
     const uint4 *codes = reinterpret_cast<const uint4 *>(a.codes) + lane;
@@ -810,19 +816,49 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
         // Rows past the end of the index or outside the allowlist get a NaN scale: their scores
         // then fail the floor compare by themselves, and the per-score path has no other test.
         if (slot0 + 32u > a.n) mw &= (a.n > slot0) ? (0xffffffffu >> (slot0 + 32u - a.n)) : 0u;
+        // the block's largest allowed row scale; a negative, huge or non-finite scale (no encoder
+        // writes such) or a largest one below 1e-30 switches the bound off for the block
+        // (the lane's query number through a move the compiler cannot see through: the addresses of
+        // its records are then formed here, per block, instead of living in registers through the stream)
+        int qrec = qn;
+        asm volatile("v_mov_b32 %0, %0" : "+v"(qrec));
+        const bool ok = (mw >> qn) & 1u;
+        float vmax = ok ? my_scale : 0.0f;
+        const bool odd = ok && !(my_scale >= 0.0f && my_scale <= 1e30f);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int i = 8 * (r >> 2) + 4 * h + (r & 3);
-            float vsr = __shfl(my_scale, i);
-            if (!((mw >> i) & 1u)) vsr = __int_as_float(0x7fc00000);
+        for (int d = 16; d >= 1; d >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, d));
+        const float inv = 1.0f / vmax;       // all scales zero: +inf, no sum reaches the bound, and every score is zero
+        const bool odd_block = __any(odd) || (vmax > 0.0f && vmax < 1e-30f);
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                const float s = fmaf(float(acc[t][r]), qs[t], qb[t]) * vsr;
-                if (s >= tau[t]) {
-                    const int q = t * kQTile + qn;
-                    const uint32_t pos = atomicAdd(&scnt[q], 1u);
-                    if (pos < kSegCap)
-                        a.cand[(size_t(q) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(s, slot0 + i);
+        for (int t = 0; t < NT; ++t) {
+            const float2 tq = s_b[t * kQTile + qrec];
+            const float bf = fmaf(tq.x, inv, -tq.y) - 1.0f;
+            int bound;
+            asm("v_cvt_i32_f32 %0, %1" : "=v"(bound) : "v"(bf));   // saturates; NaN gives 0
+            if (odd_block) bound = int(0x80000000);
+            const v16i &c = acc[t];
+            int m = max(max(c[0], c[1]), c[2]);       // (one running maximum: the kernel has no register to spare)
+            m = max(max(m, c[3]), c[4]);
+            m = max(max(m, c[5]), c[6]);
+            m = max(max(m, c[7]), c[8]);
+            m = max(max(m, c[9]), c[10]);
+            m = max(max(m, c[11]), c[12]);
+            m = max(max(m, c[13]), c[14]);
+            m = max(m, c[15]);
+            if (__any(m >= bound)) {      // (the whole wave: the row scales come from its lanes)
+                const float4 qp = s_q[t * kQTile + qrec];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int i = 8 * (r >> 2) + 4 * h + (r & 3);
+                    float vsr = __shfl(my_scale, i);
+                    if (!((mw >> i) & 1u)) vsr = __int_as_float(0x7fc00000);
+                    const float s = fmaf(float(acc[t][r]), qp.x, qp.y) * vsr;
+                    if (s >= qp.z) {
+                        const int q = t * kQTile + qn;
+                        const uint32_t pos = atomicAdd(&scnt[q], 1u);
+                        if (pos < kSegCap)
+                            a.cand[(size_t(q) * a.seg_stride + blockIdx.x) * kSegCap + pos] = sort_key(s, slot0 + i);
+                    }
                 }
             }
         }
@@ -1740,9 +1776,10 @@ hipError_t launch_scan_p4(const ScanArgs &args, int grid, int mode, hipStream_t 
 // weights through LDS in slices (k_scan_p4_batched).
 
 // Query tiles whose weights fit LDS together, capped at 4.
+constexpr size_t kMultiFixedLds = kDecodeBytes + (4 * kQTile + 4) * sizeof(uint32_t) + 4 * kQTile * 24;   // beside the weights, at four tiles
 static int resident_tiles(int nch) {
     const size_t per_tile = size_t(nch) * 2048;
-    int nt = int((kLdsBudget - 1024 - kDecodeBytes) / per_tile);
+    int nt = int((kLdsBudget - kMultiFixedLds) / per_tile);
     return nt > 4 ? 4 : nt;
 }
 
@@ -1767,7 +1804,7 @@ int batched_grid_blocks(int device, int nch) {
     if (hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0)
         cus = prop.multiProcessorCount;
     if (resident_tiles(nch) >= 2) {
-        const size_t lds = size_t(resident_tiles(nch)) * nch * 2048 + 1024 + kDecodeBytes;
+        const size_t lds = size_t(resident_tiles(nch)) * nch * 2048 + kMultiFixedLds;
         const int per_cu = int(kLdsBudget / lds);
         return cus * (per_cu < 1 ? 1 : (per_cu > 2 ? 2 : per_cu));
     }
@@ -1776,7 +1813,7 @@ int batched_grid_blocks(int device, int nch) {
 
 template <int NT, int U>
 static hipError_t launch_multi_u(const ScanArgs &a, int grid, hipStream_t s) {
-    const size_t lds = kDecodeBytes + size_t(NT) * a.nch * 2048 + (NT * kQTile + 1) * sizeof(uint32_t);
+    const size_t lds = kDecodeBytes + size_t(NT) * a.nch * 2048 + (NT * kQTile + 4) * sizeof(uint32_t) + size_t(NT) * kQTile * 24;
     hipError_t e = allow_lds(k_scan_p4_multi<NT, U, kMultiThreads<NT>>, lds);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((k_scan_p4_multi<NT, U, kMultiThreads<NT>>), dim3(grid), dim3(kMultiThreads<NT>), lds, s, a);
