@@ -1776,11 +1776,14 @@ hipError_t launch_scan_p4(const ScanArgs &args, int grid, int mode, hipStream_t 
 // weights through LDS in slices (k_scan_p4_batched).
 
 // Query tiles whose weights fit LDS together, capped at 4.
-constexpr size_t kMultiFixedLds = kDecodeBytes + (4 * kQTile + 4) * sizeof(uint32_t) + 4 * kQTile * 24;   // beside the weights, at four tiles
+// LDS of the resident-weights kernel beside nt tiles' weights: the byte table, the candidate
+// counters and the block counter, and 24 bytes of constants per query.
+static size_t multi_fixed_lds(int nt) { return kDecodeBytes + (size_t(nt) * kQTile + 4) * sizeof(uint32_t) + size_t(nt) * kQTile * 24; }
 static int resident_tiles(int nch) {
     const size_t per_tile = size_t(nch) * 2048;
-    int nt = int((kLdsBudget - kMultiFixedLds) / per_tile);
-    return nt > 4 ? 4 : nt;
+    for (int nt = 4; nt >= 1; --nt)
+        if (nt * per_tile + multi_fixed_lds(nt) <= kLdsBudget) return nt;
+    return 0;
 }
 
 // Waves per workgroup of the resident-weights kernel: three per SIMD (measured best of 512 / 768 /
@@ -1804,7 +1807,7 @@ int batched_grid_blocks(int device, int nch) {
     if (hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0)
         cus = prop.multiProcessorCount;
     if (resident_tiles(nch) >= 2) {
-        const size_t lds = size_t(resident_tiles(nch)) * nch * 2048 + kMultiFixedLds;
+        const size_t lds = size_t(resident_tiles(nch)) * nch * 2048 + multi_fixed_lds(resident_tiles(nch));
         const int per_cu = int(kLdsBudget / lds);
         return cus * (per_cu < 1 ? 1 : (per_cu > 2 ? 2 : per_cu));
     }
@@ -1813,7 +1816,7 @@ int batched_grid_blocks(int device, int nch) {
 
 template <int NT, int U>
 static hipError_t launch_multi_u(const ScanArgs &a, int grid, hipStream_t s) {
-    const size_t lds = kDecodeBytes + size_t(NT) * a.nch * 2048 + (NT * kQTile + 4) * sizeof(uint32_t) + size_t(NT) * kQTile * 24;
+    const size_t lds = size_t(NT) * a.nch * 2048 + multi_fixed_lds(NT);
     hipError_t e = allow_lds(k_scan_p4_multi<NT, U, kMultiThreads<NT>>, lds);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((k_scan_p4_multi<NT, U, kMultiThreads<NT>>), dim3(grid), dim3(kMultiThreads<NT>), lds, s, a);
