@@ -131,6 +131,19 @@ __device__ __forceinline__ uint32_t levels_of(uint32_t nib, uint32_t t0, uint32_
     return __builtin_amdgcn_perm(t1, t0, selA) & __builtin_amdgcn_perm(t3, t2, selB);
 }
 
+// Largest value of v over the wave (all 64 lanes active), in every lane: four butterfly steps inside
+// each row of 16 lanes on the data-parallel path (no LDS), then the four row results through lane
+// reads.
+__device__ __forceinline__ uint32_t wave_umax(uint32_t v) {
+    v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0xB1, 0xf, 0xf, false)));    // quad_perm [1,0,3,2]
+    v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x4E, 0xf, 0xf, false)));    // quad_perm [2,3,0,1]
+    v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x141, 0xf, 0xf, false)));   // row_half_mirror
+    v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x140, 0xf, 0xf, false)));   // row_mirror
+    const uint32_t a = uint32_t(__builtin_amdgcn_readlane(int(v), 0)), b = uint32_t(__builtin_amdgcn_readlane(int(v), 16));
+    const uint32_t c = uint32_t(__builtin_amdgcn_readlane(int(v), 32)), d = uint32_t(__builtin_amdgcn_readlane(int(v), 48));
+    return max(max(a, b), max(c, d));
+}
+
 // The code byte -> (level of its low nibble, level of its high nibble) table the permute-dot scans
 // keep at the start of their LDS: 256 entries of two int8 levels.
 constexpr int kDecodeBytes = 512;

@@ -747,6 +747,7 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
     // outside 1e-30 .. 1e30 switch the bound off for that query (every tile scored).
     float4 *s_q = reinterpret_cast<float4 *>(snext + 4);      // [NT * 32] (scale, bias, floor, -)
     float2 *s_b = reinterpret_cast<float2 *>(s_q + NT * kQTile);   // [NT * 32] (ta, tb) of the bound
+    float *s_vs = reinterpret_cast<float *>(s_b + NT * kQTile) + (tid >> 6) * 32;   // this wave's: the row scales of the block it finishes, NaN where not allowed
     for (int q = tid; q < NT * kQTile; q += THREADS) {
         scnt[q] = 0u;
         const bool act = q < a.nq_tile;
@@ -823,11 +824,11 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
         int qrec = qn;
         asm volatile("v_mov_b32 %0, %0" : "+v"(qrec));
         const bool ok = (mw >> qn) & 1u;
-        float vmax = ok ? my_scale : 0.0f;
         const bool odd = ok && !(my_scale >= 0.0f && my_scale <= 1e30f);
-#pragma unroll
-        for (int d = 16; d >= 1; d >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, d));
+        // (non-negative floats order like their bit patterns: the maximum on the data-parallel path, no LDS)
+        const float vmax = __uint_as_float(wave_umax(ok && !odd ? __float_as_uint(my_scale) : 0u));
         const float inv = 1.0f / vmax;       // all scales zero: +inf, no sum reaches the bound, and every score is zero
+        if (lane < 32) s_vs[lane] = ok ? my_scale : __int_as_float(0x7fc00000);   // for the tiles scored below (read by this wave only)
         const bool odd_block = __any(odd) || (vmax > 0.0f && vmax < 1e-30f);
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
@@ -845,14 +846,13 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
             m = max(max(m, c[11]), c[12]);
             m = max(max(m, c[13]), c[14]);
             m = max(m, c[15]);
-            if (__any(m >= bound)) {      // (the whole wave: the row scales come from its lanes)
+            if (m >= bound) {
                 const float4 qp = s_q[t * kQTile + qrec];
+                const float *vs = s_vs + 4 * h;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int i = 8 * (r >> 2) + 4 * h + (r & 3);
-                    float vsr = __shfl(my_scale, i);
-                    if (!((mw >> i) & 1u)) vsr = __int_as_float(0x7fc00000);
-                    const float s = fmaf(float(acc[t][r]), qp.x, qp.y) * vsr;
+                    const float s = fmaf(float(acc[t][r]), qp.x, qp.y) * vs[8 * (r >> 2) + (r & 3)];
                     if (s >= qp.z) {
                         const int q = t * kQTile + qn;
                         const uint32_t pos = atomicAdd(&scnt[q], 1u);
@@ -1198,18 +1198,6 @@ __global__ __launch_bounds__(256) void k_merge(const float *__restrict__ part_sc
 // redo through the list path.
 // ===========================================================================
 
-// Largest value of v over the wave (all 64 lanes active), in every lane: four butterfly steps inside
-// each row of 16 lanes on the data-parallel path (no LDS), then the four row results through lane
-// reads.
-__device__ __forceinline__ uint32_t wave_umax(uint32_t v) {
-    v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0xB1, 0xf, 0xf, false)));    // quad_perm [1,0,3,2]
-    v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x4E, 0xf, 0xf, false)));    // quad_perm [2,3,0,1]
-    v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x141, 0xf, 0xf, false)));   // row_half_mirror
-    v = max(v, uint32_t(__builtin_amdgcn_update_dpp(0, int(v), 0x140, 0xf, 0xf, false)));   // row_mirror
-    const uint32_t a = uint32_t(__builtin_amdgcn_readlane(int(v), 0)), b = uint32_t(__builtin_amdgcn_readlane(int(v), 16));
-    const uint32_t c = uint32_t(__builtin_amdgcn_readlane(int(v), 32)), d = uint32_t(__builtin_amdgcn_readlane(int(v), 48));
-    return max(max(a, b), max(c, d));
-}
 __device__ __forceinline__ uint64_t wave_umax64(uint64_t v) {
     const uint32_t hi = uint32_t(v >> 32), lo = uint32_t(v);
     const uint32_t mhi = wave_umax(hi);
@@ -1777,8 +1765,8 @@ hipError_t launch_scan_p4(const ScanArgs &args, int grid, int mode, hipStream_t 
 
 // Query tiles whose weights fit LDS together, capped at 4.
 // LDS of the resident-weights kernel beside nt tiles' weights: the byte table, the candidate
-// counters and the block counter, and 24 bytes of constants per query.
-static size_t multi_fixed_lds(int nt) { return kDecodeBytes + (size_t(nt) * kQTile + 4) * sizeof(uint32_t) + size_t(nt) * kQTile * 24; }
+// counters and the block counter, 24 bytes of constants per query, a block's row scales per wave.
+static size_t multi_fixed_lds(int nt) { return kDecodeBytes + (size_t(nt) * kQTile + 4) * sizeof(uint32_t) + size_t(nt) * kQTile * 24 + 16 * 32 * sizeof(float); }
 static int resident_tiles(int nch) {
     const size_t per_tile = size_t(nch) * 2048;
     for (int nt = 4; nt >= 1; --nt)
