@@ -876,13 +876,13 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
         if (block_ends) { pj = claim(); pc = 0; }
         const bool more = pj < nj;
         issue(nxt, nxt_sc, (more ? pj : j) * step, more ? pc : c0);
+        // the group's weights: one address per tile, the chunk and the operand as immediate offsets
+        uint32_t w_at[NT];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int c = c0 + u;
-            if (u == 0) wait_vm<2 * U - 0>(cur[0]);
-            if (u == 1) wait_vm<2 * U - 1>(cur[U > 1 ? 1 : 0]);
-            if (u == 2) wait_vm<2 * U - 2>(cur[U > 2 ? 2 : 0]);
-            if (u == 3) wait_vm<2 * U - 3>(cur[U > 3 ? 3 : 0]);
+        for (int t = 0; t < NT; ++t) w_at[t] = w_base + (uint32_t(c0) * 2048u + uint32_t(t) * w_tile);
+        static_for<U>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            wait_vm<2 * U - u>(cur[u]);
             // Split decode as in k_scan_p4: code bytes 8..15 of the lane through the byte table
             // (requested first), bytes 0..7 on the vector ALU while those reads and the first
             // operand's weights are on their way; the second operand's weights travel during the
@@ -893,11 +893,10 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
             lds_u16(e[1], byte_x2<2>(cur[u].z)); lds_u16(o[1], byte_x2<3>(cur[u].z));
             lds_u16(e[2], byte_x2<0>(cur[u].w)); lds_u16(o[2], byte_x2<1>(cur[u].w));
             lds_u16(e[3], byte_x2<2>(cur[u].w)); lds_u16(o[3], byte_x2<3>(cur[u].w));
-            const uint32_t w_addr = w_base + uint32_t(c) * 2048u;
             v4i b0[NT], b1[NT];
             static_for<NT>([&](auto tc) {
                 constexpr int t = decltype(tc)::value;
-                lds_b128_at(b0[t], w_addr + uint32_t(t) * w_tile);
+                lds_b128<u * 2048>(b0[t], w_at[t]);
             });
             const v4i a0 = {int(levels_of(cur[u].x & 0x0f0f0f0fu, t0, t1, t2, t3)),
                             int(levels_of((cur[u].x >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3)),
@@ -906,7 +905,7 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
             lds_settle_all(e, o, b0);
             static_for<NT>([&](auto tc) {
                 constexpr int t = decltype(tc)::value;
-                lds_b128_at(b1[t], w_addr + uint32_t(t) * w_tile + 1024u);
+                lds_b128<u * 2048 + 1024>(b1[t], w_at[t]);
             });
 #pragma unroll
             for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b0[t], acc[t], 0, 0, 0);
@@ -914,7 +913,7 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
             lds_settle_all(e, o, b1);
 #pragma unroll
             for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b1[t], acc[t], 0, 0, 0);
-        }
+        });
         if (block_ends) {
             wait_vm<U + 1>(cur_sc);   // this group's own scale: only the request issued above is younger
             finish_block(b, cur_sc);
