@@ -445,6 +445,13 @@ __device__ __forceinline__ void lds_settle(uint32_t (&e)[4], uint32_t (&o)[4], v
 __device__ __forceinline__ void lds_b128_at(v4i &dst, uint32_t addr) {
     asm volatile("ds_read_b128 %0, %1" : "=&v"(dst) : "v"(addr));
 }
+// (the same for two table dwords)
+template <int NT>
+__device__ __forceinline__ void lds_settle_all(uint32_t (&e)[2], uint32_t (&o)[2], v4i (&w)[NT]) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e[0]), "+v"(e[1]), "+v"(o[0]), "+v"(o[1]));
+#pragma unroll
+    for (int t = 0; t < NT; ++t) asm volatile("" : "+v"(w[t]));
+}
 template <int NT>
 __device__ __forceinline__ void lds_settle_all(uint32_t (&e)[4], uint32_t (&o)[4], v4i (&w)[NT]) {
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(e[0]), "+v"(e[1]), "+v"(e[2]), "+v"(e[3]), "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3]));
@@ -718,8 +725,13 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4(ScanArgs a) {
 // main loop.  Used when NT * dim fits the 160 KiB of LDS.
 // ===========================================================================
 
-template <int NT, int U, int THREADS>
+// LB = code bytes of a lane's sixteen that are decoded through the LDS byte table (8: bytes 8..15;
+// 4: bytes 12..15, bytes 8..11 then go through the vector ALU like bytes 0..7 and are interleaved
+// into the table's (low, high) order by two byte permutes: fewer LDS reads in flight and fewer
+// registers, which lets the three-tile instance run four waves per SIMD).
+template <int NT, int U, int THREADS, int LB>
 __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
+    static_assert(LB == 8 || LB == 4, "table bytes per lane and chunk");
     extern __shared__ __align__(16) uint8_t smem[];
     if (launch_switched_off(a.run_if)) return;
     const int nch = a.nch;
@@ -888,11 +900,14 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
             // operand's weights are on their way; the second operand's weights travel during the
             // first operand's MFMAs.  All LDS traffic of the loop is requested and waited for by
             // hand, so the counts below are exact.
-            uint32_t e[4], o[4];
-            lds_u16(e[0], byte_x2<0>(cur[u].z)); lds_u16(o[0], byte_x2<1>(cur[u].z));
-            lds_u16(e[1], byte_x2<2>(cur[u].z)); lds_u16(o[1], byte_x2<3>(cur[u].z));
-            lds_u16(e[2], byte_x2<0>(cur[u].w)); lds_u16(o[2], byte_x2<1>(cur[u].w));
-            lds_u16(e[3], byte_x2<2>(cur[u].w)); lds_u16(o[3], byte_x2<3>(cur[u].w));
+            constexpr int kTab = LB / 2;      // dwords of the second operand that come from the table (two code bytes each)
+            uint32_t e[kTab], o[kTab];
+            if constexpr (LB == 8) {
+                lds_u16(e[0], byte_x2<0>(cur[u].z)); lds_u16(o[0], byte_x2<1>(cur[u].z));
+                lds_u16(e[1], byte_x2<2>(cur[u].z)); lds_u16(o[1], byte_x2<3>(cur[u].z));
+            }
+            lds_u16(e[kTab - 2], byte_x2<0>(cur[u].w)); lds_u16(o[kTab - 2], byte_x2<1>(cur[u].w));
+            lds_u16(e[kTab - 1], byte_x2<2>(cur[u].w)); lds_u16(o[kTab - 1], byte_x2<3>(cur[u].w));
             v4i b0[NT], b1[NT];
             static_for<NT>([&](auto tc) {
                 constexpr int t = decltype(tc)::value;
@@ -902,6 +917,13 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
                             int(levels_of((cur[u].x >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3)),
                             int(levels_of(cur[u].y & 0x0f0f0f0fu, t0, t1, t2, t3)),
                             int(levels_of((cur[u].y >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3))};
+            uint32_t z01[2] = {0u, 0u};       // LB = 4: the second operand's first two dwords, from bytes 8..11
+            if constexpr (LB == 4) {
+                const uint32_t lo = levels_of(cur[u].z & 0x0f0f0f0fu, t0, t1, t2, t3);
+                const uint32_t hi = levels_of((cur[u].z >> 4) & 0x0f0f0f0fu, t0, t1, t2, t3);
+                z01[0] = __builtin_amdgcn_perm(hi, lo, 0x05010400u);      // (low, high) of byte 8, of byte 9
+                z01[1] = __builtin_amdgcn_perm(hi, lo, 0x07030602u);      // of bytes 10 and 11
+            }
             lds_settle_all(e, o, b0);
             static_for<NT>([&](auto tc) {
                 constexpr int t = decltype(tc)::value;
@@ -909,7 +931,12 @@ __global__ __launch_bounds__(THREADS) void k_scan_p4_multi(ScanArgs a) {
             });
 #pragma unroll
             for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b0[t], acc[t], 0, 0, 0);
-            const v4i a1 = {int(e[0] | (o[0] << 16)), int(e[1] | (o[1] << 16)), int(e[2] | (o[2] << 16)), int(e[3] | (o[3] << 16))};
+            v4i a1;
+            if constexpr (LB == 8) {
+                a1 = v4i{int(e[0] | (o[0] << 16)), int(e[1] | (o[1] << 16)), int(e[2] | (o[2] << 16)), int(e[3] | (o[3] << 16))};
+            } else {
+                a1 = v4i{int(z01[0]), int(z01[1]), int(e[0] | (o[0] << 16)), int(e[1] | (o[1] << 16))};
+            }
             lds_settle_all(e, o, b1);
 #pragma unroll
             for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b1[t], acc[t], 0, 0, 0);
@@ -1773,10 +1800,13 @@ static int resident_tiles(int nch) {
     return 0;
 }
 
-// Waves per workgroup of the resident-weights kernel: three per SIMD (measured best of 512 / 768 /
-// 1024 threads with three and four tiles' accumulators); the two-tile instance fits 128 registers
-// and runs four per SIMD (2 to 7 % faster per launch, 256 to 2048 dimensions).
-template <int NT> constexpr int kMultiThreads = NT == 2 ? 1024 : 768;
+// Waves per workgroup of the resident-weights kernel and code bytes per lane and chunk it decodes
+// through the table.  Four tiles: three waves per SIMD (measured best of 512 / 768 / 1024 threads),
+// eight table bytes.  Two tiles fit 128 registers and run four waves per SIMD (2 to 7 % faster per
+// launch, 256 to 2048 dimensions).  Three tiles fit them with four table bytes -- fewer reads in
+// flight, fewer registers; by itself that split is 1 % slower -- and gain 1 to 3 % from the fourth wave.
+template <int NT> constexpr int kMultiTableBytes = NT == 3 ? 4 : 8;
+template <int NT> constexpr int kMultiThreads = NT <= 3 ? 1024 : 768;
 constexpr int kStreamTiles = 4, kStreamBlocksPerWave = 2, kStreamSliceChunks = 2, kStreamOccupancy = 2;
 
 // The resident-weights kernel reads its weights in k_scan_p4's split order.
@@ -1803,10 +1833,11 @@ int batched_grid_blocks(int device, int nch) {
 
 template <int NT, int U>
 static hipError_t launch_multi_u(const ScanArgs &a, int grid, hipStream_t s) {
+    constexpr int LB = kMultiTableBytes<NT>;
     const size_t lds = size_t(NT) * a.nch * 2048 + multi_fixed_lds(NT);
-    hipError_t e = allow_lds(k_scan_p4_multi<NT, U, kMultiThreads<NT>>, lds);
+    hipError_t e = allow_lds(k_scan_p4_multi<NT, U, kMultiThreads<NT>, LB>, lds);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((k_scan_p4_multi<NT, U, kMultiThreads<NT>>), dim3(grid), dim3(kMultiThreads<NT>), lds, s, a);
+    hipLaunchKernelGGL((k_scan_p4_multi<NT, U, kMultiThreads<NT>, LB>), dim3(grid), dim3(kMultiThreads<NT>), lds, s, a);
     return hipGetLastError();
 }
 
