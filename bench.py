@@ -34,9 +34,9 @@ sys.path.insert(0, ROOT)
 # HBM bytes one launch of the dominant kernel moves (reads + writes), from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this same command, each scaled by the copy-probe factor (see profiles/).
 MEASURED_TRAFFIC = {
-    ("k_scan_p4_wide", 10_000_000, 1536, 4): 7.7826e9,    # 3,775,910 x 2 KiB fetched + 48,417 KiB written
-    ("k_scan_p4_multi", 10_000_000, 1536, 4): 7.7361e9,   # 3,775,700 x 2 KiB fetched + 3,396 KiB written
-    ("k_scan_p4", 10_000_000, 1536, 4): 7.7208e9,         # 3,769,800 x 2 KiB fetched + 270 KiB written
+    ("k_scan_p4_wide", 10_000_000, 1536, 4): 7.7826e9,    # 3,775,910 x 2 KiB fetched + 48,384 KiB written
+    ("k_scan_p4_multi", 10_000_000, 1536, 4): 7.7359e9,   # 3,775,570 x 2 KiB fetched + 3,451 KiB written
+    ("k_scan_p4", 10_000_000, 1536, 4): 7.7208e9,         # 3,769,800 x 2 KiB fetched + 265 KiB written
     ("k_scan_lut_bt", 10_000_000, 1536, 2): 3.8802e9,     # 1,894,650 x 2 KiB fetched
     ("k_scan_lut16", 10_000_000, 1536, 2): 3.8830e9,      # 1,895,400 x 2 KiB fetched + 1,189 KiB written
     ("k_scan_lut", 10_000_000, 1536, 2): 3.8809e9,        # 1,894,970 x 2 KiB fetched
